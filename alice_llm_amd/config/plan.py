@@ -32,13 +32,16 @@ class LayerPlan:
 
     `norms` is keyed by the role the block gives each norm, e.g. "pre_mixer",
     "post_mixer", "pre_ff", "post_ff"; a block uses the roles it knows and
-    treats an absent one as no norm at that place.
+    treats an absent one as no norm at that place.  `feed_forward` may be None (a layer without one, for
+    arrangements that allow it).  `extras` are further parts of the layer, keyed by the role the block gives
+    them (a per-layer token input, say), each from the EXTRAS registry.
     """
     block: str
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]
     norms: Mapping[str, PartSpec]
     prefix: str
+    extras: Mapping[str, PartSpec] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -46,9 +49,11 @@ class ScheduleEntry:
     """One run of a layer.  Every run owns cache storage of its own (a layer named twice keeps two
     caches, one per run), unless `cache_from` names an earlier entry of the schedule, by its index,
     whose cache this run reads instead of writing one (the reference's kv_layer_map,
-    llama3.rs:4739-4745)."""
+    llama3.rs:4739-4745).  `before` names one of the plan's shared parts (a stream operation) that acts on
+    the residual stream right before this run."""
     layer: int
     cache_from: Optional[int] = None
+    before: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -63,6 +68,9 @@ class ModelPlan:
     final_norm: PartSpec
     head: PartSpec
     stop_token_ids: Tuple[int, ...] = ()
+    # parts that belong to the model and not to one layer, by name: tables that several layers read, operations
+    # on the residual stream between layers.  Each from the SHARED registry; its tensors are named `name.local`.
+    shared: Mapping[str, PartSpec] = field(default_factory=dict)
 
 
 # --------------------------------------------------------------------------- typed reads

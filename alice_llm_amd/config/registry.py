@@ -17,7 +17,7 @@ _MODEL_TYPES: Dict[str, str] = {}
 
 
 def register_architecture(name: str, config_cls: type, model_type: str = None) -> None:
-    """Register a configuration class under config.json's `architectures[0]` name.
+    """Register a configuration class under config.json's `architectures[0]` (or `architecture`) name.
 
     The class needs `from_dict(mapping)`, `to_dict()` and `plan() -> ModelPlan`.
     """
@@ -37,10 +37,12 @@ def architecture_name(d: Mapping[str, Any]) -> str:
     archs = d.get("architectures")
     if isinstance(archs, (list, tuple)) and archs and isinstance(archs[0], str):
         name = archs[0]
+    elif isinstance(d.get("architecture"), str):
+        name = d["architecture"]
     elif isinstance(d.get("model_type"), str) and d["model_type"] in _MODEL_TYPES:
         name = _MODEL_TYPES[d["model_type"]]
     else:
-        raise ConfigError("config.json: neither 'architectures' nor a known 'model_type' names the "
+        raise ConfigError("config.json: neither 'architectures', 'architecture' nor a known 'model_type' names the "
                           f"architecture; registered: {registered_architectures()}")
     if name not in _ARCHITECTURES:
         raise ConfigError(f"config.json: unknown architecture '{name}'; "

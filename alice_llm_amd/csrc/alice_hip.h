@@ -4,10 +4,11 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 6
+#define ALICE_ABI_VERSION 7
 
 #define ALICE_EPI_NONE 0
-#define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked, y = gelu_tanh(gate x) * (up x)
+#define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked; epi_param 0: y = gelu_tanh(gate x) * (up x); epi_param = limit > 0:
+                              // g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1)
 #define ALICE_EPI_SOFTCAP 2   // y = cap * tanh(y / cap)
 #define ALICE_EPI_ROPE 3      // internal: rotation and cache write (alice_linear_rope_cache)
 
@@ -64,11 +65,12 @@ int alice_linear_split_hint(int M, int N, int K, int w_layout);
 int alice_to_frag16(const void* src, void* dst, int N, int K, hipStream_t stream);
 int alice_frag16_supported(int rows, int K, int epilogue);
 
+// dv: the size of a value head (the v part of a row holds nKV * dv elements, the value pool's rows dv); 0: d.
 int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, void* k_pool, void* v_pool,
                            const float* cos_t, const float* sin_t, const int* positions,
                            const int* seq_of_token, const int* block_table, int bt_stride, int T,
                            int row_width, int nH, int nKV, int d, int rotary_dim, int page_size, int n_pages,
-                           int kv_layout, int interleaved, hipStream_t stream);
+                           int kv_layout, int interleaved, int dv, hipStream_t stream);
 
 // The fused q|k|v projection with the rotation and the cache write as its epilogue (single tokens: the
 // streaming kernel; more than 64 tokens: the tiled one): x [M, K] (row-major or fragment order), W in the fragment layout with the rows of every q and k
@@ -81,11 +83,14 @@ int alice_linear_rope_cache(const void* x, int x_layout, const void* w, int M, i
 
 // bias_slopes: null, or nH floats: head h's capped score of key k for the query at position p gets
 // bias_slopes[h] * (k - p) added before the softmax (a linear distance bias at the score stage).
+// dv: the size of a value head (0: d); out is [T, nH * dv].  gate: null, or the tokens' rows of gate_stride
+// elements (the dtype of q) whose first nH hold one number a head: head h's output is multiplied by
+// sigmoid(gate[t * gate_stride + h]).
 int alice_attention_generic(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
                             const int* positions, const int* seq_of_token, const int* block_table,
                             int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
                             float softcap, int window, const float* bias_slopes, int full_precision,
-                            hipStream_t stream);
+                            int dv, const void* gate, int gate_stride, hipStream_t stream);
 
 // bfloat16 attention on the matrix cores over a cache in the fragment layout (kv_layout 1 of
 // alice_rope_cache_write): prompts, and single tokens with the keys split over `splits` blocks.
@@ -110,6 +115,22 @@ int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool
 int alice_linear_parts_split(int M, int N, int nH, int d, int splits);
 int alice_linear_parts(const float* parts, int splits, int nH, int d, const void* w, float* y, int M, int N,
                        hipStream_t stream);
+
+// The matrix memory (mLSTM), one step or several per sequence, with the head norm, its weight and the output
+// gate behind it (see mlstm.hip).  proj: float32 rows [q: H*d | k: H*d | v: H*dv | g: H*dv | a: H | b: H] of
+// row_w numbers; bias_i, bias_f: float32 [H]; norm_w: [H*dv]; out: [T, H*dv]; sequence s owns the rows
+// cu_seqlens[s] .. cu_seqlens[s+1] and the state rows slots[s] of S [n_slots, H, d, dv], n [n_slots, H, d] and
+// m [n_slots, H], all float32.
+int alice_mlstm_step(const float* proj, int row_w, const float* bias_i, const float* bias_f,
+                     const void* norm_w, int norm_dtype, void* out, int out_dtype,
+                     const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
+                     int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, hipStream_t stream);
+
+// out[t, j] = gelu_tanh(z[t, j]) * table[tokens[t], col0 + j], j < n: a gate on columns of a per-token table
+// [V, table_w]; a token outside the table reads zeros.
+int alice_gelu_mul_rows(const void* z, int z_dtype, const void* table, int table_dtype, int table_w, int col0,
+                        const int* tokens, void* out, int out_dtype, int T, int n, int V,
+                        int full_precision, hipStream_t stream);
 
 // Lowest index among equal maxima.
 int alice_argmax_chunks(int B, int V);

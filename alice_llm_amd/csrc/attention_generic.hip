@@ -23,7 +23,8 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pool, const T* __restrict__ v_pool, T* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int bt_stride, int nH, int nKV, int d, int page_size,
-    float scale, float cap, int window, int DG, const float* __restrict__ bias_slopes) {
+    float scale, float cap, int window, int DG, const float* __restrict__ bias_slopes,
+    int dv, const T* __restrict__ gate, int gate_stride) {
   __shared__ float qs[256];
   __shared__ float sc[CHUNK];
   __shared__ float red[17];
@@ -71,11 +72,11 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
     l_run = l_run * corr + block_sum(lsum, red);      // the barriers inside also publish sc[]
     m_run = m_new;
     acc *= corr;
-    if (j < d) {
+    if (j < dv) {
       for (int i = g; i < n; i += G) {
         const int kp = c0 + i;
         const int page = bt[kp / page_size];
-        const T* vrow = v_pool + (((size_t)page * nKV + kvh) * page_size + kp % page_size) * d;
+        const T* vrow = v_pool + (((size_t)page * nKV + kvh) * page_size + kp % page_size) * dv;
         acc = fmaf(sc[i], load_f32(vrow, j), acc);
       }
     }
@@ -83,10 +84,12 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
   }
   part[tid] = acc;
   __syncthreads();
-  if (tid < d) {
+  if (tid < dv) {
     float o = 0.f;
     for (int gg = 0; gg < G; ++gg) o += part[gg * DG + tid];
-    store_f32(out + ((size_t)t * nH + h) * d, tid, o / l_run);
+    o /= l_run;
+    if (gate) o *= sigmoid_f(load_f32(gate, (size_t)t * gate_stride + h), FULL);
+    store_f32(out + ((size_t)t * nH + h) * dv, tid, o);
   }
 }
 
@@ -96,7 +99,10 @@ extern "C" int alice_attention_generic(const void* q, int dtype, const void* k_p
                                        const int* positions, const int* seq_of_token, const int* block_table,
                                        int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
                                        float softcap, int window, const float* bias_slopes, int full_precision,
-                                       hipStream_t stream) {
+                                       int dv, const void* gate, int gate_stride, hipStream_t stream) {
+  if (dv <= 0) dv = d;
+  ALICE_CHECK(dv <= 256, "attention: value head size %d is outside 1..256, the range of this kernel", dv);
+  ALICE_CHECK(gate == nullptr || gate_stride >= nH, "attention: gate rows of %d elements are too short for %d heads", gate_stride, nH);
   ALICE_CHECK(dtype_ok(dtype), "attention: unknown dtype %d", dtype);
   ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 1 && nH % nKV == 0, "attention: bad head counts nH=%d nKV=%d", nH, nKV);
   ALICE_CHECK(d >= 1 && d <= 256, "attention: head_dim %d is outside 1..256, the range of this kernel", d);
@@ -105,15 +111,15 @@ extern "C" int alice_attention_generic(const void* q, int dtype, const void* k_p
   ALICE_CHECK(softcap >= 0.f && window >= 0, "attention: softcap and window must not be negative (0 turns them off)");
   if (T == 0) return 0;
   int DG = 1;
-  while (DG < d) DG <<= 1;
+  while (DG < dv) DG <<= 1;
   dim3 grid(T, nH);
   DISPATCH_DTYPE(dtype, TT, {
     if (full_precision)
       attn_generic_kernel<TT, true><<<grid, THREADS, 0, stream>>>((const TT*)q, (const TT*)k_pool, (const TT*)v_pool,
-          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG, bias_slopes);
+          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG, bias_slopes, dv, (const TT*)gate, gate_stride);
     else
       attn_generic_kernel<TT, false><<<grid, THREADS, 0, stream>>>((const TT*)q, (const TT*)k_pool, (const TT*)v_pool,
-          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG, bias_slopes);
+          (TT*)out, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, page_size, scale, softcap, window, DG, bias_slopes, dv, (const TT*)gate, gate_stride);
   });
   ALICE_LAUNCH_CHECK();
   return 0;

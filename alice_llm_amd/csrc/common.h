@@ -102,6 +102,20 @@ __device__ __forceinline__ float gelu_tanh_f(float z, bool full) {
   return 0.5f * z * (1.f + t);
 }
 
+// The gated product of two stacked matrices' outputs (gate g, up u), the epilogue ALICE_EPI_GEGLU.  Its
+// parameter picks the form: 0 gives gelu_tanh(g) * u; a positive `limit` gives the limited form
+// g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1).
+__device__ __forceinline__ float gated_act(float g, float u, float limit, bool full) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    const float e = full ? expf(-1.702f * g) : __expf(-1.702f * g);
+    return g * (u + 1.f) / (1.f + e);
+  }
+  return gelu_tanh_f(g, full) * u;
+}
+__device__ __forceinline__ float sigmoid_f(float z, bool full) { return 1.f / (1.f + (full ? expf(-z) : __expf(-z))); }
+
 // ---- host side -------------------------------------------------------------------------
 void alice_set_error(const char* fmt, ...);
 

@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void linear_tiled_kernel(const TA* __restrict_
         const int n = n0 + tx * 2 + j;
         if (n < N) {
           float g = acc[i][j], u = acc[i][j + 2];
-          store_f32(Y, (size_t)m * N + n, gelu_tanh_f(g, FULL) * u);
+          store_f32(Y, (size_t)m * N + n, gated_act(g, u, epi, FULL));
         }
       }
     } else {
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(const TA* __restrict__
     for (int r = 0; r < NR; ++r) v[r] = wave_sum(acc[r][m]);
     if (lane == 0) {
       float o = v[0];
-      if (EPI == ALICE_EPI_GEGLU) o = gelu_tanh_f(v[0], FULL) * v[NR - 1];
+      if (EPI == ALICE_EPI_GEGLU) o = gated_act(v[0], v[NR - 1], epi, FULL);
       if (EPI == ALICE_EPI_SOFTCAP) o = epi * (FULL ? tanh_full(o / epi) : tanh_fast(o / epi));
       store_f32(Y, (size_t)m * N + n, o);
     }

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16_t* __
         const int n = (blockIdx.x * (RT / 2) + p) * 16 + g * 4;
         f32x4 o;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = gelu_tanh_f(acc[2 * p][j][i], FULL) * acc[2 * p + 1][j][i];
+        for (int i = 0; i < 4; ++i) o[i] = gated_act(acc[2 * p][j][i], acc[2 * p + 1][j][i], epi, FULL);
         if constexpr (sizeof(TO) == 2) {
           if (y_frag) { if (n < N) store4_frag((bf16_t*)yo, row[j], n, N, o); continue; }
         }

@@ -321,7 +321,7 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_lds_kernel(const bf16_t* 
         const int n = tile[2 * p] * 16 + g * 4;
         f32x4 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_f(acc[2 * p][j][e], FULL) * acc[2 * p + 1][j][e];
+        for (int e = 0; e < 4; ++e) o[e] = gated_act(acc[2 * p][j][e], acc[2 * p + 1][j][e], epi, FULL);
         store4_any(y, y_frag, m, row_off, n, N, o);
       }
     } else {

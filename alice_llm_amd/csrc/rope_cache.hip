@@ -21,7 +21,7 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
                                   const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                   const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                                   const int* __restrict__ block_table, int bt_stride, int row_w,
-                                  int nH, int nKV, int d, int R, int page_size, int n_pages, int layout, int interleaved) {
+                                  int nH, int nKV, int d, int R, int page_size, int n_pages, int layout, int interleaved, int dv) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = R >> 1;
@@ -35,12 +35,11 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
   if (k_pool) {
     const int page = block_table[(size_t)seq_of_token[t] * bt_stride + pos / page_size];
     if (page >= 0 && page < n_pages) {
-      const size_t base = (size_t)page * nKV * page_size * d;
-      kdst = k_pool + base;
-      vdst = v_pool + base;
+      kdst = k_pool + (size_t)page * nKV * page_size * d;
+      vdst = v_pool + (size_t)page * nKV * page_size * dv;
     }
   }
-  const int hd2 = d >> 1;        // work items per head: one per pair of the first/second half
+  const int hd2 = d > 1 ? d >> 1 : 1;   // work items per head: one per pair of the first/second half
   // blockIdx.y names the head this block handles: q heads, then k heads, then v heads.
   const int h = blockIdx.y;
   if (h < nH + nKV) {
@@ -63,9 +62,9 @@ __global__ void rope_cache_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
     }
   } else if (vdst) {
     const int hv = h - nH - nKV;
-    const T* vsrc = row + (size_t)(nH + nKV + hv) * d;
-    T* dst = vdst + (size_t)hv * page_size * d;
-    for (int e = threadIdx.x; e < d; e += blockDim.x) dst[v_offset(layout, tp, e, d)] = vsrc[e];
+    const T* vsrc = row + (size_t)(nH + nKV) * d + (size_t)hv * dv;
+    T* dst = vdst + (size_t)hv * page_size * dv;
+    for (int e = threadIdx.x; e < dv; e += blockDim.x) dst[v_offset(layout, tp, e, dv)] = vsrc[e];
   }
 }
 
@@ -167,10 +166,11 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
                                       const float* cos_t, const float* sin_t, const int* positions,
                                       const int* seq_of_token, const int* block_table, int bt_stride,
                                       int T, int row_width, int nH, int nKV, int d, int rotary_dim, int page_size,
-                                      int n_pages, int kv_layout, int interleaved, hipStream_t stream) {
+                                      int n_pages, int kv_layout, int interleaved, int dv, hipStream_t stream) {
+  if (dv <= 0) dv = d;
   ALICE_CHECK(dtype_ok(dtype), "rope: unknown dtype %d", dtype);
   ALICE_CHECK(!interleaved || (rotary_dim == d && cos_t != nullptr), "rope: interleaved pairs need the whole head rotated");
-  ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 0 && d >= 2 && d % 2 == 0, "rope: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
+  ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 0 && d >= 1 && (d % 2 == 0 || rotary_dim == 0), "rope: bad sizes T=%d nH=%d nKV=%d d=%d", T, nH, nKV, d);
   ALICE_CHECK(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0, "rope: rotated width %d must be even and at most head_dim %d", rotary_dim, d);
   ALICE_CHECK((cos_t == nullptr) == (sin_t == nullptr), "rope: cos and sin tables must come together");
   ALICE_CHECK(rotary_dim == 0 || cos_t != nullptr, "rope: a rotated width needs the tables");
@@ -178,12 +178,12 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
   ALICE_CHECK(k_pool == nullptr || (block_table && seq_of_token && page_size > 0 && n_pages > 0 && nKV >= 1),
               "rope: a cache write needs the block table, the token-to-sequence map and the page geometry");
   ALICE_CHECK(nH + 2 * nKV <= 65535, "rope: too many heads for one launch");
-  ALICE_CHECK(row_width >= (nH + (k_pool ? 2 * nKV : 0)) * d, "rope: rows of %d elements are too short for the heads", row_width);
-  ALICE_CHECK(kv_layout == 0 || (kv_layout == 1 && page_size == 64 && d % 32 == 0 && dtype == DT_BF16) || k_pool == nullptr,
+  ALICE_CHECK(row_width >= (nH + (k_pool ? nKV : 0)) * d + (k_pool ? nKV * dv : 0), "rope: rows of %d elements are too short for the heads", row_width);
+  ALICE_CHECK(kv_layout == 0 || (kv_layout == 1 && page_size == 64 && d % 32 == 0 && dv % 32 == 0 && dtype == DT_BF16) || k_pool == nullptr,
               "rope: the fragment cache layout needs bfloat16, pages of 64 and head_dim %% 32 == 0");
   if (T == 0) return 0;
   // Many tokens: the vector kernel (a block per token).  Few: a block per token and head has more in flight.
-  if (T >= 256 && dtype == DT_BF16 && rotary_dim == d && d % 16 == 0 && row_width % 8 == 0 && cos_t != nullptr &&
+  if (T >= 256 && dtype == DT_BF16 && rotary_dim == d && dv == d && d % 16 == 0 && row_width % 8 == 0 && cos_t != nullptr &&
       ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)q_out & 15) == 0 && ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0 &&
       (k_pool == nullptr || (((uintptr_t)k_pool & 15) == 0 && ((uintptr_t)v_pool & 15) == 0))) {
     const int items = (nH + nKV) * (d / 16) + nKV * (d / 8);
@@ -195,7 +195,7 @@ extern "C" int alice_rope_cache_write(const void* qkv, int dtype, void* q_out, v
   }
   DISPATCH_DTYPE(dtype, TT, (rope_cache_kernel<TT><<<dim3(T, nH + (k_pool ? 2 * nKV : 0)), d >= 256 ? 128 : 64, 0, stream>>>(
       (const TT*)qkv, (TT*)q_out, (TT*)k_pool, (TT*)v_pool, cos_t, sin_t, positions, seq_of_token,
-      block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages, kv_layout, interleaved)));
+      block_table, bt_stride, row_width, nH, nKV, d, rotary_dim, page_size, n_pages, kv_layout, interleaved, dv)));
   ALICE_LAUNCH_CHECK();
   return 0;
 }

@@ -10,19 +10,35 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..config.plan import ModelPlan, PartSpec
-from ..parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, ParamSpec, Precision,
-                     ResidualStream)
+from ..parts import (BLOCKS, EMBEDDINGS, EXTRAS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, SHARED, ParamSpec,
+                     Precision, ResidualStream)
+
+
+def full_name(prefix: str, local: str) -> str:
+    """A tensor's name from its part's prefix ("l0.norm1.") and the part's local name; a part whose one
+    tensor carries the part's own name declares the local name "" (the tensor is then "l0.norm1")."""
+    return prefix + local if local else prefix[:-1]
 
 
 class Layer:
-    def __init__(self, plan_layer, precision: Precision, positions: dict):
+    def __init__(self, plan_layer, precision: Precision, positions: dict, shared: dict = None):
         self.prefix = plan_layer.prefix
         self.mixer = MIXERS.get(plan_layer.mixer.kind)(precision, positions, **plan_layer.mixer.args)
-        self.feed_forward = FEED_FORWARDS.get(plan_layer.feed_forward.kind)(precision, **plan_layer.feed_forward.args)
+        ff = plan_layer.feed_forward
+        self.feed_forward = None if ff is None else FEED_FORWARDS.get(ff.kind)(precision, **ff.args)
         self.norms = {role: NORMS.get(spec.kind)(precision, **spec.args) for role, spec in plan_layer.norms.items()}
-        self.block = BLOCKS.get(plan_layer.block)(self.mixer, self.feed_forward, self.norms)
-        self._named = [(plan_layer.mixer.name, self.mixer), (plan_layer.feed_forward.name, self.feed_forward)]
+        # further parts of the layer (a per-layer token input, say); they may read the model's shared parts
+        self.extras = {role: EXTRAS.get(spec.kind)(precision, shared or {}, **spec.args)
+                       for role, spec in plan_layer.extras.items()}
+        if self.extras or self.feed_forward is None:
+            self.block = BLOCKS.get(plan_layer.block)(self.mixer, self.feed_forward, self.norms, self.extras)
+        else:
+            self.block = BLOCKS.get(plan_layer.block)(self.mixer, self.feed_forward, self.norms)
+        self._named = [(plan_layer.mixer.name, self.mixer)]
+        if ff is not None:
+            self._named.append((ff.name, self.feed_forward))
         self._named += [(plan_layer.norms[role].name, n) for role, n in self.norms.items()]
+        self._named += [(plan_layer.extras[role].name, e) for role, e in self.extras.items()]
 
     def named_parts(self):
         return [(self.prefix + name + ".", part) for name, part in self._named]
@@ -39,12 +55,16 @@ class CausalLM:
         if "none" not in self.positions:
             self.positions["none"] = POSITIONS.get("none")(p, self.device)
         self.embedding = EMBEDDINGS.get(plan.embedding.kind)(p, **plan.embedding.args)
-        self.layers: List[Layer] = [Layer(lp, p, self.positions) for lp in plan.layers]
+        # parts of the model that belong to no single layer: tables that layers share, stream operations
+        self.shared = {name: SHARED.get(spec.kind)(p, **spec.args) for name, spec in plan.shared.items()}
+        self.layers: List[Layer] = [Layer(lp, p, self.positions, self.shared) for lp in plan.layers]
         self.final_norm = NORMS.get(plan.final_norm.kind)(p, **plan.final_norm.args) if plan.final_norm else None
         self.head = HEADS.get(plan.head.kind)(p, **plan.head.args)
         for i, e in enumerate(plan.schedule):
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"schedule entry {i} names layer {e.layer}, which does not exist")
+            if e.before is not None and not hasattr(self.shared.get(e.before), "apply"):
+                raise ValueError(f"schedule entry {i} names the stream operation '{e.before}', which the plan does not share")
             if e.cache_from is not None:
                 if not 0 <= e.cache_from < i or plan.schedule[e.cache_from].cache_from is not None:
                     raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache_from}, which must be "
@@ -60,6 +80,7 @@ class CausalLM:
     # ------------------------------------------------------------------ parameters
     def named_parts(self) -> List[Tuple[str, object]]:
         out = [(self.plan.embedding.name + ".", self.embedding)]
+        out += [(name + ".", part) for name, part in self.shared.items()]
         for layer in self.layers:
             out += layer.named_parts()
         if self.final_norm is not None:
@@ -72,13 +93,17 @@ class CausalLM:
         specs: "OrderedDict[str, ParamSpec]" = OrderedDict()
         for prefix, part in self.named_parts():
             for local, spec in part.param_specs().items():
-                specs[prefix + local] = spec
+                specs[full_name(prefix, local)] = spec
         return specs
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
         for prefix, part in self.named_parts():
-            if name.startswith(prefix) and name[len(prefix):] in part.param_specs():
+            specs = part.param_specs()
+            if name.startswith(prefix) and name[len(prefix):] in specs:
                 part.assign(name[len(prefix):], tensor)
+                return
+            if name == prefix[:-1] and "" in specs:
+                part.assign("", tensor)
                 return
         raise KeyError(name)
 
@@ -105,9 +130,9 @@ class CausalLM:
     def graph_safe(self) -> bool:
         """Whether a decode step of this model can be recorded into a HIP graph: every part that runs in a
         step declares `graph_safe = True` (its launches depend on device data and on sizes fixed per graph)."""
-        parts = [self.embedding, self.head, self.final_norm] + list(self.positions.values())
+        parts = [self.embedding, self.head, self.final_norm] + list(self.positions.values()) + list(self.shared.values())
         for layer in self.layers:
-            parts += [layer.mixer, layer.feed_forward, layer.block] + list(layer.norms.values())
+            parts += [layer.mixer, layer.feed_forward, layer.block] + list(layer.norms.values()) + list(layer.extras.values())
         return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
 
     def prompt_graph_safe(self) -> bool:
@@ -135,7 +160,11 @@ class CausalLM:
         if not self._loaded:
             raise RuntimeError("the model has no weights yet")
         stream = ResidualStream(self.embedding.forward(ctx), self.precision)
+        if any(e.before is not None for e in self.plan.schedule):
+            stream.start = stream.x.clone()            # the embedding output, for stream operations that read it
         for i, entry in enumerate(self.plan.schedule):
+            if entry.before is not None:
+                self.shared[entry.before].apply(stream, ctx)
             view = cache.view(i, block_tables, read_from=entry.cache_from)
             self.layers[entry.layer].block.forward(stream, ctx, view)
         if ctx.want_rows is None or ctx.want_rows.numel() == 0:

@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _lib = None
 _lib_path = None
@@ -43,12 +43,14 @@ def _declare(lib) -> None:
         "alice_linear_split_hint": [I, I, I, I],
         "alice_to_frag16": [P, P, I, I, P],
         "alice_frag16_supported": [I, I, I],
-        "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, P],
+        "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, I, P],
+        "alice_mlstm_step": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, F, F, P],
+        "alice_gelu_mul_rows": [P, I, P, I, I, I, P, P, I, I, I, I, I, P],
         "alice_linear_rope_cache": [P, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
-        "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, P],
+        "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
@@ -294,8 +296,10 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
                      v_pool: Optional[torch.Tensor], cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                      positions: torch.Tensor, seq_of_token: Optional[torch.Tensor],
                      block_table: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int, head_dim: int,
-                     rotary_dim: int, max_position: int, kv_layout: int = 0, interleaved: bool = False) -> None:
-    """Rotate q and k; write k and v at their positions into the pools [pages, nKV, page, d].
+                     rotary_dim: int, max_position: int, kv_layout: int = 0, interleaved: bool = False,
+                     value_head_dim: Optional[int] = None) -> None:
+    """Rotate q and k; write k and v at their positions into the pools [pages, nKV, page, d]
+    (values [pages, nKV, page, value_head_dim] where that differs from d).
     With k_pool None the row holds q only (num_kv_heads = 0) and nothing is cached.
     `max_position` is the largest position among `positions` (the host knows it): checked against the tables.
     interleaved: the q and k heads of qkv hold the rotated pairs (j, j + d/2) at 2j and 2j + 1 (a projection
@@ -304,7 +308,8 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
     dt = qkv.dtype
     _dev(qkv, "qkv")
     row_width = qkv.shape[1]
-    if qkv.dim() != 2 or row_width < (num_heads + (2 * num_kv_heads if k_pool is not None else 0)) * head_dim:
+    dv = head_dim if value_head_dim is None else int(value_head_dim)
+    if qkv.dim() != 2 or row_width < num_heads * head_dim + (num_kv_heads * (head_dim + dv) if k_pool is not None else 0):
         raise HipLibraryError(f"qkv rows of {tuple(qkv.shape)} are too short for the heads")
     _dev(q_out, "q_out", dt, (T, num_heads * head_dim))
     _dev(positions, "positions", torch.int32, (T,))
@@ -320,7 +325,7 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
         if k_pool.dim() != 4 or k_pool.shape[1] != num_kv_heads or k_pool.shape[3] != head_dim:
             raise HipLibraryError(f"k_pool must be [pages, {num_kv_heads}, page, {head_dim}], found {tuple(k_pool.shape)}")
         _dev(k_pool, "k_pool", dt)
-        _dev(v_pool, "v_pool", dt, k_pool.shape)
+        _dev(v_pool, "v_pool", dt, tuple(k_pool.shape[:3]) + (dv,))
         n_pages, _, page_size, _ = k_pool.shape
         _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
         _dev(block_table, "block_table", torch.int32)
@@ -332,7 +337,7 @@ def rope_cache_write(qkv: torch.Tensor, q_out: torch.Tensor, k_pool: Optional[to
     _call("alice_rope_cache_write", qkv.data_ptr(), dtype_code(dt), q_out.data_ptr(), _opt(k_pool, "k_pool"),
           _opt(v_pool, "v_pool"), _opt(cos, "cos"), _opt(sin, "sin"), positions.data_ptr(),
           _opt(seq_of_token, "seq_of_token"), _opt(block_table, "block_table"), bt_stride, T, row_width, num_heads,
-          num_kv_heads, head_dim, rotary_dim, page_size, n_pages, int(kv_layout), int(interleaved), _stream())
+          num_kv_heads, head_dim, rotary_dim, page_size, n_pages, int(kv_layout), int(interleaved), dv, _stream())
 
 
 def linear_rope_cache(x: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
@@ -382,18 +387,28 @@ def linear_rope_cache(x: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, k_p
 def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor,
                       positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, *,
                       num_heads: int, scale: float, softcap: Optional[float], window: Optional[int],
-                      max_position: int, full_precision: bool, bias_slopes: Optional[torch.Tensor] = None) -> None:
+                      max_position: int, full_precision: bool, bias_slopes: Optional[torch.Tensor] = None,
+                      gate: Optional[torch.Tensor] = None) -> None:
     """bias_slopes: float32 [num_heads]; head h's capped score of key k for the query at position p gets
-    bias_slopes[h] * (k - p) added before the softmax."""
+    bias_slopes[h] * (k - p) added before the softmax.  The value pool's last size is the value head size
+    (out: [T, heads * that]).  gate: [T, >= num_heads] in q's dtype, rows of any stride (a column slice of a
+    wider tensor): head h's output is multiplied by sigmoid(gate[t, h])."""
     T = q.shape[0]
     dt = q.dtype
-    if k_pool.dim() != 4:
+    if k_pool.dim() != 4 or v_pool.dim() != 4:
         raise HipLibraryError("k_pool must be [pages, nKV, page, d]")
     n_pages, nKV, page_size, d = k_pool.shape
+    dv = v_pool.shape[3]
     _dev(q, "q", None, (T, num_heads * d))
-    _dev(out, "out", dt, (T, num_heads * d))
+    _dev(out, "out", dt, (T, num_heads * dv))
     _dev(k_pool, "k_pool", dt)
-    _dev(v_pool, "v_pool", dt, k_pool.shape)
+    _dev(v_pool, "v_pool", dt, tuple(k_pool.shape[:3]) + (dv,))
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        if (not gate.is_cuda or gate.dtype != dt or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < num_heads
+                or gate.stride(1) != 1 or gate.stride(0) < num_heads):
+            raise HipLibraryError(f"gate must be [{T}, >= {num_heads}] {dt} with unit column stride")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
     _dev(positions, "positions", torch.int32, (T,))
     _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
     _dev(block_table, "block_table", torch.int32)
@@ -405,7 +420,7 @@ def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
           out.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
           block_table.shape[1], T, num_heads, nKV, d, page_size, float(scale),
           float(softcap or 0.0), int(window or 0), None if bias_slopes is None else bias_slopes.data_ptr(),
-          int(full_precision), _stream())
+          int(full_precision), int(dv), gate_ptr, int(gate_stride), _stream())
 
 
 def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:
@@ -535,14 +550,15 @@ def linear_parts(parts: torch.Tensor, splits: int, w: torch.Tensor, y: torch.Ten
 def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: torch.Tensor, ctx,
               block_table: torch.Tensor, *, num_heads: int, scale: float, softcap: Optional[float],
               window: Optional[int], full_precision: bool, kv_layout: int = KV_ROW,
-              out_layout: int = LAYOUT_ROW, bias_slopes: Optional[torch.Tensor] = None) -> None:
+              out_layout: int = LAYOUT_ROW, bias_slopes: Optional[torch.Tensor] = None,
+              gate: Optional[torch.Tensor] = None) -> None:
     """Attention of the step's query tokens over the cache; picks the kernel for the step's shape and
     the cache's layout.  `ctx` carries positions, seq_of_token, cu_seqlens, context_lens and the
     host-side sizes of the step.  out_layout FRAG16 is taken by the matrix-core kernels only; a score bias
     (bias_slopes, see attention_generic) by the generic kernel only, over a row-major cache."""
     if kv_layout == KV_FRAGMENT:
-        if bias_slopes is not None:
-            raise HipLibraryError("the matrix-core attention kernels take no score bias: lay the cache out row-major")
+        if bias_slopes is not None or gate is not None:
+            raise HipLibraryError("the matrix-core attention kernels take no score bias and no gate: lay the cache out row-major")
         nKV = k_pool.shape[1]
         if ctx.is_decode and num_heads // nKV <= 16:
             attention_decode(q, k_pool, v_pool, out, ctx.context_lens, block_table, num_heads=num_heads,
@@ -558,7 +574,60 @@ def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: 
         raise HipLibraryError("only the matrix-core attention kernels write fragment order")
     attention_generic(q, k_pool, v_pool, out, ctx.positions, ctx.seq_of_token, block_table,
                       num_heads=num_heads, scale=scale, softcap=softcap, window=window,
-                      max_position=ctx.max_position, full_precision=full_precision, bias_slopes=bias_slopes)
+                      max_position=ctx.max_position, full_precision=full_precision, bias_slopes=bias_slopes, gate=gate)
+
+
+MLSTM_MAX_VALUE_DIM = 1024      # the largest value head size the matrix-memory kernels take
+
+
+def mlstm(proj, bias_i, bias_f, norm_w, out, ctx, S, n, m, *, heads: int, head_dim: int, value_head_dim: int,
+          cap: float, eps: float) -> None:
+    """The matrix memory over a step; picks the kernel for the step's shape (see mlstm_step)."""
+    mlstm_step(proj, bias_i, bias_f, norm_w, out, ctx.cu_seqlens, ctx.slots, S, n, m, n_seqs=ctx.n_seqs, heads=heads,
+               head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
+
+
+def mlstm_step(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, norm_w: torch.Tensor, out: torch.Tensor,
+               cu_seqlens: torch.Tensor, slots: torch.Tensor, S: torch.Tensor, n: torch.Tensor, m: torch.Tensor, *,
+               n_seqs: int, heads: int, head_dim: int, value_head_dim: int, cap: float, eps: float) -> None:
+    """The matrix memory over the step's tokens, sequence by sequence from the state rows slots[s], with the head
+    norm, its weight and the output gate behind it.  proj: float32 [T, >= 2 H d + 2 H dv + 2 H] rows
+    [q | k | v | g | a | b]; out: [T, H dv] in the activation dtype; S [slots, H, d, dv], n [slots, H, d],
+    m [slots, H] float32."""
+    H, d, dv = heads, head_dim, value_head_dim
+    T = proj.shape[0]
+    _dev(proj, "proj", torch.float32)
+    if proj.dim() != 2 or proj.shape[1] < 2 * H * d + 2 * H * dv + 2 * H:
+        raise HipLibraryError(f"proj rows of {tuple(proj.shape)} are too short")
+    _dev(bias_i, "bias_i", torch.float32, (H,))
+    _dev(bias_f, "bias_f", torch.float32, (H,))
+    _dev(norm_w, "norm_w", None, (H * dv,))
+    _dev(out, "out", None, (T, H * dv))
+    _dev(cu_seqlens, "cu_seqlens", torch.int32)
+    _dev(slots, "slots", torch.int32)
+    if cu_seqlens.numel() < n_seqs + 1 or slots.numel() < n_seqs:
+        raise HipLibraryError("cu_seqlens and slots are too short for the step's sequences")
+    n_slots = S.shape[0]
+    _dev(S, "S", torch.float32, (n_slots, H, d, dv))
+    _dev(n, "n", torch.float32, (n_slots, H, d))
+    _dev(m, "m", torch.float32, (n_slots, H))
+    _call("alice_mlstm_step", proj.data_ptr(), proj.shape[1], bias_i.data_ptr(), bias_f.data_ptr(), norm_w.data_ptr(),
+          dtype_code(norm_w.dtype), out.data_ptr(), dtype_code(out.dtype), cu_seqlens.data_ptr(), slots.data_ptr(),
+          S.data_ptr(), n.data_ptr(), m.data_ptr(), int(n_seqs), int(n_slots), H, d, dv, float(cap), float(eps), _stream())
+
+
+def gelu_mul_rows(z: torch.Tensor, table: torch.Tensor, col0: int, tokens: torch.Tensor, out: torch.Tensor, *,
+                  full_precision: bool) -> None:
+    """out[t, j] = gelu_tanh(z[t, j]) * table[tokens[t], col0 + j]; table: row-major [V, width]."""
+    T, n = z.shape
+    _dev(z, "z")
+    _dev(out, "out", z.dtype, (T, n))
+    _dev(tokens, "tokens", torch.int32)
+    if tokens.numel() < T or table.dim() != 2:
+        raise HipLibraryError("gelu_mul_rows: one token per row and a [V, width] table")
+    _dev(table, "table")
+    _call("alice_gelu_mul_rows", z.data_ptr(), dtype_code(z.dtype), table.data_ptr(), dtype_code(table.dtype), table.shape[1],
+          int(col0), tokens.data_ptr(), out.data_ptr(), dtype_code(out.dtype), T, n, table.shape[0], int(full_precision), _stream())
 
 
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

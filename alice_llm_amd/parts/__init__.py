@@ -1,5 +1,5 @@
-from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, CacheNeed, FragmentActs, KVNeed,
-                   ParamSpec, Part, Precision, Registry, StateNeed)
+from .base import (BLOCKS, EMBEDDINGS, EXTRAS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITIONS, SHARED, CacheNeed,
+                   FragmentActs, KVNeed, ParamSpec, Part, Precision, Registry, StateNeed)
 from .linear import Linear
 from .stream import ResidualStream
-from . import norm, rope, attention, feedforward, embedding, block  # noqa: F401  (register the parts)
+from . import norm, rope, attention, feedforward, embedding, block, mlstm, composite, token_input, stream_ops  # noqa: F401  (register the parts)

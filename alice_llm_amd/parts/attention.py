@@ -8,7 +8,10 @@ counts and head size are constructor arguments; window None is global attention,
 turns the tanh off.  A position term at the score stage is a constructor argument too:
 score_bias_slopes, one slope a query head, adds slope * (key position - query position) to the
 capped score (a linear distance bias; the 32-bit attention kernel over a row-major cache takes it,
-in both dtypes).
+in both dtypes).  Values may have a head size of their own (value_head_dim), and output_gate = "head" adds
+one gate number a query head, projected from the mixer's input beside q, k and v: head h's output is
+multiplied by sigmoid(gate_h) before the output projection.  tensor_names gives the local names of the
+matrices (q, k, v, o, g) where a file names them otherwise.
 """
 from __future__ import annotations
 
@@ -28,7 +31,8 @@ class Attention(Part):
     def __init__(self, precision: Precision, positions: dict, *, hidden_size: int, num_heads: int,
                  num_kv_heads: int, head_dim: int, scale: float, softcap: Optional[float] = None,
                  window: Optional[int] = None, position: Optional[str] = None,
-                 score_bias_slopes: Optional[Sequence[float]] = None):
+                 score_bias_slopes: Optional[Sequence[float]] = None, value_head_dim: Optional[int] = None,
+                 output_gate: Optional[str] = None, tensor_names: Optional[Dict[str, str]] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_kv_heads {num_kv_heads} must divide num_heads {num_heads}")
         if not 1 <= head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
@@ -47,45 +51,61 @@ class Attention(Part):
         self.position = positions[position] if position is not None else positions.get("none")
         if self.position is None:
             raise ValueError("attention needs a position encoding (use 'none' for no rotation)")
-        self.q_dim, self.kv_dim = num_heads * head_dim, num_kv_heads * head_dim
-        self.qkv = Linear(hidden_size, self.q_dim + 2 * self.kv_dim, precision)
-        self.o = Linear(self.q_dim, hidden_size, precision)
+        self.dv = head_dim if value_head_dim is None else int(value_head_dim)
+        if not 1 <= self.dv <= ops.ATTENTION_MAX_HEAD_DIM:
+            raise ValueError(f"attention: value_head_dim {self.dv} is outside 1..{ops.ATTENTION_MAX_HEAD_DIM}")
+        if output_gate not in (None, "head"):
+            raise ValueError(f"attention: output_gate '{output_gate}' is not known (None or 'head')")
+        self.output_gate = output_gate
+        self.n_gate = num_heads if output_gate == "head" else 0
+        self.names = dict({"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                           "g": "g_proj.weight"}, **(tensor_names or {}))
+        self.q_dim, self.kv_dim, self.v_dim = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * self.dv
+        self.o_in = num_heads * self.dv
+        # one fused projection: all q heads, the k heads, the v heads, then the gate numbers
+        self.qkv = Linear(hidden_size, self.q_dim + self.kv_dim + self.v_dim + self.n_gate, precision)
+        self.o = Linear(self.o_in, hidden_size, precision)
         # How this mixer lays keys and values out inside a page: the matrix-core kernels read a fragment
         # layout; every other case is row-major.  It depends on the arithmetic and the head size alone, so
         # that a run that reads another run's cache finds the layout it expects.
         self.kv_layout = (ops.KV_FRAGMENT if precision.name == "bfloat16" and precision.act == torch.bfloat16
                           and ops.library_ready() and ops.attention_mfma_supported(head_dim)
-                          and score_bias_slopes is None else ops.KV_ROW)
+                          and score_bias_slopes is None and self.dv == head_dim and not self.n_gate else ops.KV_ROW)
         self._parts: Dict[str, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"q_proj.weight": ParamSpec((self.q_dim, self.H)),
-                "k_proj.weight": ParamSpec((self.kv_dim, self.H)),
-                "v_proj.weight": ParamSpec((self.kv_dim, self.H)),
-                "o_proj.weight": ParamSpec((self.H, self.q_dim))}
+        n = self.names
+        specs = {n["q"]: ParamSpec((self.q_dim, self.H)),
+                 n["k"]: ParamSpec((self.kv_dim, self.H)),
+                 n["v"]: ParamSpec((self.v_dim, self.H)),
+                 n["o"]: ParamSpec((self.H, self.o_in))}
+        if self.n_gate:
+            specs[n["g"]] = ParamSpec((self.n_gate, self.H))
+        return specs
 
     def cache_need(self) -> CacheNeed:
         # the fragment layout of the matrix-core kernels is written for pages of 64 positions
         page = ops.KV_FRAGMENT_PAGE if self.kv_layout == ops.KV_FRAGMENT else None
-        return CacheNeed(kv=KVNeed(self.nKV, self.d, self.window, page_size=page))
+        return CacheNeed(kv=KVNeed(self.nKV, self.d, self.window, page_size=page,
+                                   value_head_dim=None if self.dv == self.d else self.dv))
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
-        if name == "o_proj.weight":
+        if name == self.names["o"]:
             self.o.load(tensor)
-        elif name in ("q_proj.weight", "k_proj.weight", "v_proj.weight"):
+        elif name in [self.names[c] for c in ("qkvg" if self.n_gate else "qkv")]:
             self._parts[name] = tensor
         else:
             raise KeyError(name)
 
     def finalize(self) -> None:
-        q, k, v = (self.precision.matrix(self._parts.pop(n + "_proj.weight")) for n in "qkv")
-        if not (q.dtype == k.dtype == v.dtype):
-            q, k, v = q.float(), k.float(), v.float()       # kept as stored, one of them in 32-bit: the fused matrix is 32-bit
-        w = torch.cat([q, k, v], dim=0)                     # rows: all q heads, then k heads, then v heads
+        mats = [self.precision.matrix(self._parts.pop(self.names[c])) for c in ("qkvg" if self.n_gate else "qkv")]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]                # kept as stored, one of them in 32-bit: the fused matrix is 32-bit
+        w = torch.cat(mats, dim=0)                          # rows: all q heads, then k heads, then v heads, then the gates
         # a position encoding may ask for the rows of the q and k heads in another order (rotated pairs next to
         # each other), so that its rotation can be the projection's epilogue
         order = getattr(self.position, "projection_row_order", lambda *a: None)(self.nH, self.nKV, self.d)
-        self.pair_order = order is not None
+        self.pair_order = order is not None and self.dv == self.d and not self.n_gate
         if self.pair_order:
             w = w[order.to(w.device)]
         self.qkv.load(w)
@@ -105,9 +125,15 @@ class Attention(Part):
         T = x.shape[0]
         q = torch.empty((T, self.q_dim), dtype=self.precision.act, device=x.device)
         geometry = dict(num_heads=self.nH, num_kv_heads=self.nKV, head_dim=self.d, kv_layout=self.kv_layout)
+        if self.dv != self.d:
+            geometry["value_head_dim"] = self.dv
+        gate = None
         fused = self.pair_order and self.position.project_rotate_store(self.qkv, x, q, ctx, cache, **geometry)
         if not fused:
             qkv = self.qkv(x, self.precision.act)
+            if self.n_gate:
+                g0 = self.q_dim + self.kv_dim + self.v_dim
+                gate = qkv[:, g0:g0 + self.n_gate]          # a column slice: the kernel reads it with the rows' stride
             if self.pair_order:
                 self.position.rotate_and_store(qkv, q, ctx, cache, pair_order=True, **geometry)
             else:
@@ -127,10 +153,11 @@ class Attention(Part):
                 return y if slices > 1 else y[0]
         # The matrix-core kernels' output goes to the output projection in fragment order.
         frag = (getattr(ctx, "fragment_activations", False) and self.kv_layout == ops.KV_FRAGMENT
-                and self.o.accepts_fragment_input and FragmentActs.possible(self.precision, T, self.q_dim))
-        out = FragmentActs.empty(T, self.q_dim, q.device) if frag else torch.empty_like(q)
+                and self.o.accepts_fragment_input and FragmentActs.possible(self.precision, T, self.o_in))
+        out = (FragmentActs.empty(T, self.o_in, q.device) if frag
+               else torch.empty((T, self.o_in), dtype=q.dtype, device=q.device))
         ops.attention(q, cache.k, cache.v, out.data if frag else out, ctx, cache.block_table, num_heads=self.nH,
                       scale=self.scale, softcap=self.softcap, window=self.window, full_precision=self.precision.full,
                       kv_layout=self.kv_layout, out_layout=ops.LAYOUT_FRAG16 if frag else ops.LAYOUT_ROW,
-                      bias_slopes=self._slopes)
+                      bias_slopes=self._slopes, gate=gate)
         return self.o(out, torch.float32, allow_partials=True)

@@ -188,3 +188,5 @@ POSITIONS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("output head")
+EXTRAS = Registry("layer extra")            # further parts of a layer: cls(precision, shared, **args)
+SHARED = Registry("shared part")            # parts of the model that belong to no single layer: cls(precision, **args)

@@ -3,6 +3,11 @@
 "sandwich": x += post_mixer(mixer(pre_mixer(x))); x += post_ff(ff(pre_ff(x))), each norm optional
 (llama3.rs:14178, 14460-14470, 14497, 14543-14557: Gemma 2 has all four; a pre-norm-only layer
 leaves the post norms out and is the same wiring).
+
+"parallel": one norm, whose output feeds the mixer and the feed-forward side by side:
+h = pre(x); x += mixer(h) + ff(h) (the feed-forward may be absent); then the layer's extras act on the
+stream in their order (a per-layer token input, say).  A mixer may return several branches, each with a post
+norm of its own.
 """
 from __future__ import annotations
 
@@ -32,3 +37,28 @@ class SandwichBlock:
 
 
 BLOCKS.register("prenorm", SandwichBlock)
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock:
+    def __init__(self, mixer, feed_forward, norms: Dict[str, object], extras: Dict[str, object] = None):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norms = norms
+        self.extras = dict(extras or {})
+
+    @property
+    def graph_safe(self) -> bool:
+        return True
+
+    def forward(self, stream, ctx, cache) -> None:
+        h = stream.normed(self.norms.get("pre"))
+        branches = self.mixer.forward(h, ctx, cache)
+        if not isinstance(branches, list):
+            branches = [(branches, None)]
+        if self.feed_forward is not None:
+            branches.append((self.feed_forward.forward(h, ctx), None))
+        for branch, post in branches:
+            stream.push(branch, post)
+        for extra in self.extras.values():
+            extra.forward(stream, ctx)

@@ -20,16 +20,18 @@ from .linear import Linear
 class Embedding(Part):
     graph_safe = True
 
-    def __init__(self, precision: Precision, *, vocab_size: int, dim: int, scale: float = 1.0):
+    def __init__(self, precision: Precision, *, vocab_size: int, dim: int, scale: float = 1.0,
+                 tensor_name: str = "weight"):
+        self.tensor_name = tensor_name
         self.precision = precision
         self.V, self.dim, self.scale = vocab_size, dim, float(scale)
         self.table = Linear(dim, vocab_size, precision)     # stored as the head reads it
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.V, self.dim))}
+        return {self.tensor_name: ParamSpec((self.V, self.dim))}
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
-        if name != "weight":
+        if name != self.tensor_name:
             raise KeyError(name)
         self.table.load(tensor)
 
@@ -51,7 +53,8 @@ class OutputHead(Part):
     graph_safe = True
 
     def __init__(self, precision: Precision, *, vocab_size: int, dim: int, softcap: Optional[float] = None,
-                 tied_to: Optional[str] = None):
+                 tied_to: Optional[str] = None, tensor_name: str = "weight"):
+        self.tensor_name = tensor_name
         self.precision = precision
         self.V, self.dim = vocab_size, dim
         self.softcap = None if softcap is None else float(softcap)
@@ -61,10 +64,10 @@ class OutputHead(Part):
                            epi_param=self.softcap or 0.0)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {} if self.tied_to else {"weight": ParamSpec((self.V, self.dim))}
+        return {} if self.tied_to else {self.tensor_name: ParamSpec((self.V, self.dim))}
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
-        if name != "weight" or self.tied_to:
+        if name != self.tensor_name or self.tied_to:
             raise KeyError(name)
         self.proj.load(tensor)
 

@@ -1,11 +1,12 @@
 """Feed-forwards.  Gated MLP: down( act(gate x) * (up x) ), the activation on the gate branch
 (llama3.rs:14519-14540); for Gemma 2 the activation is the tanh form of GELU
-(llama3.rs:6183-6186).  gate and up are stacked into one matrix at load so that one kernel reads
+(llama3.rs:6183-6186).  A second gated form, "swish_limited", bounds both branches first:
+g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1).  gate and up are stacked into one matrix at load so that one kernel reads
 the input once and applies the activation and the product in its epilogue.
 """
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
@@ -13,38 +14,47 @@ from ..hip import ops
 from .base import FEED_FORWARDS, ParamSpec, Part, Precision
 from .linear import Linear
 
-_GATED_EPILOGUES = {"gelu_tanh": ops.EPI_GEGLU}
+# both forms are the gated epilogue of the matrix products; its parameter picks the form (0: tanh-GELU times up;
+# a positive limit: the limited swish form)
+_GATED_EPILOGUES = {"gelu_tanh": ops.EPI_GEGLU, "swish_limited": ops.EPI_GEGLU}
+_DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
 
 @FEED_FORWARDS.register("gated_mlp")
 class GatedMLP(Part):
     graph_safe = True
 
-    def __init__(self, precision: Precision, *, hidden_size: int, intermediate_size: int, activation: str):
+    def __init__(self, precision: Precision, *, hidden_size: int, intermediate_size: int, activation: str,
+                 limit: Optional[float] = None, tensor_names: Optional[Dict[str, str]] = None):
         if activation not in _GATED_EPILOGUES:
             raise ValueError(f"gated_mlp has no kernel for activation '{activation}'; "
                              f"available: {sorted(_GATED_EPILOGUES)}")
+        if (activation == "swish_limited") != (limit is not None) or (limit is not None and not limit > 0):
+            raise ValueError("gated_mlp: 'swish_limited' takes a positive limit, and only it does")
         self.precision = precision
         self.H, self.I = hidden_size, intermediate_size
-        self.gate_up = Linear(hidden_size, intermediate_size, precision, epilogue=_GATED_EPILOGUES[activation])
+        self.names = dict(_DEFAULT_NAMES, **(tensor_names or {}))
+        self.gate_up = Linear(hidden_size, intermediate_size, precision, epilogue=_GATED_EPILOGUES[activation],
+                              epi_param=float(limit or 0.0))
         self.down = Linear(intermediate_size, hidden_size, precision)
         self._parts: Dict[str, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"gate_proj.weight": ParamSpec((self.I, self.H)),
-                "up_proj.weight": ParamSpec((self.I, self.H)),
-                "down_proj.weight": ParamSpec((self.H, self.I))}
+        n = self.names
+        return {n["gate"]: ParamSpec((self.I, self.H)),
+                n["up"]: ParamSpec((self.I, self.H)),
+                n["down"]: ParamSpec((self.H, self.I))}
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
-        if name == "down_proj.weight":
+        if name == self.names["down"]:
             self.down.load(tensor)
-        elif name in ("gate_proj.weight", "up_proj.weight"):
+        elif name in (self.names["gate"], self.names["up"]):
             self._parts[name] = tensor
         else:
             raise KeyError(name)
 
     def finalize(self) -> None:
-        g, u = (self.precision.matrix(self._parts.pop(n + "_proj.weight")) for n in ("gate", "up"))
+        g, u = (self.precision.matrix(self._parts.pop(self.names[n])) for n in ("gate", "up"))
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         self.gate_up.load(torch.cat([g, u], dim=0))

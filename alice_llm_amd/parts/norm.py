@@ -2,7 +2,8 @@
 
 The reference multiplies by the stored weight (llama3.rs:5244-5256), its files holding 1 + w; a
 safetensors file holds w, so Gemma 2 passes weight_offset = 1.  The offset, eps and the width are
-constructor arguments: another convention is another argument value.
+constructor arguments: another convention is another argument value.  `tensor_name` is the weight's local
+name ("" where the tensor carries the part's own name).
 """
 from __future__ import annotations
 
@@ -18,7 +19,9 @@ from .base import NORMS, ParamSpec, Part, Precision
 class RMSNorm(Part):
     graph_safe = True
 
-    def __init__(self, precision: Precision, *, dim: int, eps: float, weight_offset: float = 0.0):
+    def __init__(self, precision: Precision, *, dim: int, eps: float, weight_offset: float = 0.0,
+                 tensor_name: str = "weight"):
+        self.tensor_name = tensor_name
         self.precision = precision
         self.dim = dim
         self.eps = float(eps)
@@ -26,10 +29,10 @@ class RMSNorm(Part):
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.dim,), init_std=0.1)}
+        return {self.tensor_name: ParamSpec((self.dim,), init_std=0.1)}
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
-        if name != "weight":
+        if name != self.tensor_name:
             raise KeyError(name)
         self.weight = tensor.contiguous()
 

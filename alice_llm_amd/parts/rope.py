@@ -50,21 +50,23 @@ class RotaryEncoding(Part):
         return torch.cat([heads.flatten(), torch.arange(v0, v0 + num_kv_heads * head_dim)])
 
     def rotate_and_store(self, qkv: torch.Tensor, q_out: torch.Tensor, ctx, cache, *, num_heads: int,
-                         num_kv_heads: int, head_dim: int, kv_layout: int = 0, pair_order: bool = False) -> None:
+                         num_kv_heads: int, head_dim: int, kv_layout: int = 0, pair_order: bool = False,
+                         value_head_dim: Optional[int] = None) -> None:
         write = cache is not None and cache.writable
         ops.rope_cache_write(qkv, q_out, cache.k if write else None, cache.v if write else None,
                              self.cos, self.sin, ctx.positions, ctx.seq_of_token if write else None,
                              cache.block_table if write else None, num_heads=num_heads,
                              num_kv_heads=num_kv_heads, head_dim=head_dim, rotary_dim=self.rotary_dim,
-                             max_position=ctx.max_position, kv_layout=kv_layout, interleaved=pair_order)
+                             max_position=ctx.max_position, kv_layout=kv_layout, interleaved=pair_order,
+                             value_head_dim=value_head_dim)
 
     def project_rotate_store(self, proj, x, q_out: torch.Tensor, ctx, cache, *, num_heads: int, num_kv_heads: int,
-                             head_dim: int, kv_layout: int) -> bool:
+                             head_dim: int, kv_layout: int, value_head_dim: Optional[int] = None) -> bool:
         """Projection (a Linear in the fragment layout with its rows in pair order), rotation and cache write as
         one kernel.  False where that kernel does not apply; the caller then takes the steps apart."""
         from .base import FragmentActs
         frag_in = isinstance(x, FragmentActs)
-        if not (cache is not None and cache.writable
+        if not (cache is not None and cache.writable and value_head_dim in (None, head_dim)
                 and proj.layout == ops.LAYOUT_FRAG16 and proj.precision.act == torch.bfloat16 and head_dim % 16 == 0
                 and (kv_layout == ops.KV_ROW or head_dim % 32 == 0)):
             return False
@@ -85,10 +87,11 @@ class NoPositionEncoding(Part):
     def __init__(self, precision: Precision, device, **_):
         pass
 
-    def rotate_and_store(self, qkv, q_out, ctx, cache, *, num_heads, num_kv_heads, head_dim, kv_layout=0) -> None:
+    def rotate_and_store(self, qkv, q_out, ctx, cache, *, num_heads, num_kv_heads, head_dim, kv_layout=0,
+                         value_head_dim=None) -> None:
         write = cache is not None and cache.writable
         ops.rope_cache_write(qkv, q_out, cache.k if write else None, cache.v if write else None, None, None,
                              ctx.positions, ctx.seq_of_token if write else None,
                              cache.block_table if write else None, num_heads=num_heads,
                              num_kv_heads=num_kv_heads, head_dim=head_dim, rotary_dim=0,
-                             max_position=ctx.max_position, kv_layout=kv_layout)
+                             max_position=ctx.max_position, kv_layout=kv_layout, value_head_dim=value_head_dim)
