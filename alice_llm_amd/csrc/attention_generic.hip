@@ -101,11 +101,11 @@ extern "C" int alice_attention_generic(const void* q, int dtype, const void* k_p
                                        float softcap, int window, const float* bias_slopes, int full_precision,
                                        int dv, const void* gate, int gate_stride, hipStream_t stream) {
   if (dv <= 0) dv = d;
-  ALICE_CHECK(dv <= 256, "attention: value head size %d is outside 1..256, the range of this kernel", dv);
   ALICE_CHECK(gate == nullptr || gate_stride >= nH, "attention: gate rows of %d elements are too short for %d heads", gate_stride, nH);
   ALICE_CHECK(dtype_ok(dtype), "attention: unknown dtype %d", dtype);
   ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 1 && nH % nKV == 0, "attention: bad head counts nH=%d nKV=%d", nH, nKV);
   ALICE_CHECK(d >= 1 && d <= 256, "attention: head_dim %d is outside 1..256, the range of this kernel", d);
+  ALICE_CHECK(dv <= 256, "attention: value head size %d is outside 1..256, the range of this kernel", dv);
   ALICE_CHECK(nH <= 65535, "attention: too many heads for one launch (%d)", nH);
   ALICE_CHECK(page_size > 0 && bt_stride > 0, "attention: bad page geometry");
   ALICE_CHECK(softcap >= 0.f && window >= 0, "attention: softcap and window must not be negative (0 turns them off)");

@@ -582,8 +582,15 @@ MLSTM_MAX_VALUE_DIM = 1024      # the largest value head size the matrix-memory 
 
 def mlstm(proj, bias_i, bias_f, norm_w, out, ctx, S, n, m, *, heads: int, head_dim: int, value_head_dim: int,
           cap: float, eps: float) -> None:
-    """The matrix memory over a step; picks the kernel for the step's shape (see mlstm_step)."""
-    mlstm_step(proj, bias_i, bias_f, norm_w, out, ctx.cu_seqlens, ctx.slots, S, n, m, n_seqs=ctx.n_seqs, heads=heads,
+    """The matrix memory over a step: `ctx` carries cu_seqlens, slots and the host-side sizes (see mlstm_rows)."""
+    mlstm_rows(proj, bias_i, bias_f, norm_w, out, ctx.cu_seqlens, ctx.slots, S, n, m, n_seqs=ctx.n_seqs,
+               max_new=ctx.max_new, heads=heads, head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
+
+
+def mlstm_rows(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, *, n_seqs: int, max_new: int, heads: int,
+               head_dim: int, value_head_dim: int, cap: float, eps: float) -> None:
+    """Picks the kernel for the step's shape: token by token for single tokens and short pieces."""
+    mlstm_step(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
                head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
 
 

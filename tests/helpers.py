@@ -130,3 +130,77 @@ def model_from_tensors(cfg, tensors, dtype):
         lm.assign(name, tensors[name])
     lm.finalize()
     return Model(cfg, lm)
+
+
+# ------------------------------------------------------------------ Novotar: three small configurations
+def _nv_layer(left, right, mlp):
+    return {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp}
+
+
+# A: a loop in the middle run twice, a token-side input, grouped kv heads, value heads twice the key size, a window
+#    shorter than a page, one layer without a feed-forward.
+# B: no loop, no token-side input, kv heads = heads, value size = key size, a window longer than a page, value heads
+#    of the matrix memory that fit no tile (40), eps and embedding scale other than A's, limits that never bind.
+# C: sizes that suit the matrix cores, a loop over every layer run three times, one kv head, window 100.
+def _nv_a():
+    le = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.3, "mask": {"size": 5}}
+    ri = {"heads": 2, "dim": 16, "vdim": 32, "gate_cap": 8.0}
+    mlp = {"kind": "dense", "ff": 96, "limit": 1.5}
+    return {"architecture": "Novotar", "vocab": 97, "width": 64, "embedding": {"scale": 4.0}, "norm": {"eps": 1e-6},
+            "layers": [_nv_layer(le, ri, mlp), _nv_layer(le, ri, None), _nv_layer(dict(le, mask={"size": 9}), ri, mlp)],
+            "loop": {"start": 1, "stop": 3, "times": 2}, "token_side": {"dim": 8}}
+
+
+def _nv_b():
+    le = {"heads": 3, "kv_heads": 3, "dim": 24, "vdim": 24, "scale": 0.2, "mask": {"size": 70}}
+    ri = {"heads": 3, "dim": 8, "vdim": 40, "gate_cap": 15.0}
+    mlp = {"kind": "dense", "ff": 80, "limit": 50.0}
+    return {"architecture": "Novotar", "vocab": 130, "width": 96, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+            "layers": [_nv_layer(le, ri, mlp), _nv_layer(le, dict(ri, heads=1, dim=32, vdim=16), mlp)]}
+
+
+def _nv_c():
+    le = {"heads": 4, "kv_heads": 1, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 100}}
+    ri = {"heads": 2, "dim": 64, "vdim": 128, "gate_cap": 10.0}
+    mlp = {"kind": "dense", "ff": 256, "limit": 3.0}
+    return {"architecture": "Novotar", "vocab": 300, "width": 128, "embedding": {"scale": 8.0}, "norm": {"eps": 1e-6},
+            "layers": [_nv_layer(le, ri, mlp), _nv_layer(le, ri, mlp)],
+            "loop": {"start": 0, "stop": 2, "times": 3}, "token_side": {"dim": 16}}
+
+
+NOVOTAR = {"nv-a": _nv_a, "nv-b": _nv_b, "nv-c": _nv_c}
+
+
+def novotar_tensors(raw: dict, seed: int):
+    """Random tensors for a Novotar configuration, by name, in bfloat16 on the CPU: matrices N(0, gain^2 / inputs) with
+    gains that make every mechanism matter (gates that open and close, limits that bind, scores of order 1), norm
+    weights around 1."""
+    import alice_llm_amd as alice
+    from alice_llm_amd.engine.model import CausalLM
+    from alice_llm_amd.parts import Precision
+    cfg = alice.config_from_dict(raw)
+    specs = CausalLM(cfg.plan(), Precision.of("float32"), "cpu").param_specs()
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, spec in specs.items():
+        shape = tuple(spec.shape)
+        r = torch.randn(shape, generator=g)
+        if len(shape) == 1:
+            t = r if name.endswith(".b") else 1.0 + 0.2 * r
+        elif name in ("embed", "side.embed"):
+            t = r * (0.5 if name == "embed" else 1.0)
+        else:
+            gain = 3.0 if name.endswith((".i", ".f", "left.q", "left.k", "left.g")) else 1.0
+            t = r * gain / shape[1] ** 0.5
+        out[name] = t.to(torch.bfloat16)
+    return cfg, out
+
+
+def novotar_pair(name: str, dtype: str, seed: int = 0, device="cuda"):
+    """(the package's model, the plain model) on the same tensors."""
+    from plain.novotar_plain import PlainNovotar
+    raw = NOVOTAR[name]()
+    cfg, tensors = novotar_tensors(raw, seed)
+    plain = PlainNovotar(raw, {k: v.double() for k, v in tensors.items()})
+    model = model_from_tensors(cfg, {k: v.to(device) for k, v in tensors.items()}, dtype)
+    return model, plain
