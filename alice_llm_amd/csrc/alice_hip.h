@@ -126,6 +126,14 @@ int alice_mlstm_step(const float* proj, int row_w, const float* bias_i, const fl
                      const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
                      int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, hipStream_t stream);
 
+// The same for steps of many tokens a sequence, a chunk of tokens at a time on the 32-bit matrix instruction;
+// work: float32 [T, H * dv].  alice_mlstm_chunks_supported says whether the head sizes are covered.
+int alice_mlstm_chunks_supported(int n_seqs, int H, int d, int dv);
+int alice_mlstm_chunks(const float* proj, int row_w, const float* bias_i, const float* bias_f,
+                       const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
+                       const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
+                       int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, hipStream_t stream);
+
 // out[t, j] = gelu_tanh(z[t, j]) * table[tokens[t], col0 + j], j < n: a gate on columns of a per-token table
 // [V, table_w]; a token outside the table reads zeros.
 int alice_gelu_mul_rows(const void* z, int z_dtype, const void* table, int table_dtype, int table_w, int col0,

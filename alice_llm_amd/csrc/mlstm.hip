@@ -136,6 +136,224 @@ __global__ void gelu_mul_rows_kernel(const TZ* __restrict__ z, const TW* __restr
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------ chunks
+// The same recurrence for many tokens of a sequence, a chunk of C tokens at a time.  Inside a chunk, with
+// b_j the running sum of the log forget gates, a_r = i_r - b_r and M_j = max(m_0, max_{r <= j} a_r) (m_0: the
+// stabiliser before the chunk), the token-by-token definition gives m_j = b_j + M_j and
+//   S_j = exp(m_0 - M_j) S_0 + sum_{r <= j} exp(a_r - M_j) k_r v_r^T          (n_j alike),
+// so that  S_j^T q_j = exp(m_0 - M_j) (Q S_0)_j + ((Q K^T . D) V)_j  with  D_jr = exp(a_r - M_j), r <= j.
+// Four matrix products a chunk (Q K^T, Q S_0, P V, K'^T V), all on the 32-bit matrix instruction
+// (v_mfma_f32_16x16x4_f32): the state, the gates' weights and everything they multiply stay 32-bit.
+// A block owns VS of a head's value columns (S's columns are independent of each other) for all chunks of
+// one sequence; blocks of one head recompute its gates and Q K^T.  The head norm needs every column, so the
+// read-outs go to a 32-bit workspace and mlstm_finish_kernel norms, weights and gates them.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int lds_pad20(int d) { return d + ((84 - d % 64) % 64); }   // stride = 20 mod 64 banks
+
+template <int C, int VS>
+__global__ __launch_bounds__(THREADS) void mlstm_chunk_kernel(
+    const float* __restrict__ proj, int row_w, const float* __restrict__ bias_i, const float* __restrict__ bias_f,
+    float* __restrict__ work, const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
+    float* __restrict__ S_all, float* __restrict__ n_all, float* __restrict__ m_all,
+    int H, int d, int dv, float cap) {
+  constexpr int VSS = VS == 32 ? 48 : 80;      // row stride of V and S tiles: 16 mod 64 banks
+  constexpr int PSS = C + 4;
+  constexpr int CT = C / 16, VT = VS / 16;
+  extern __shared__ float lds[];
+  const int QS = lds_pad20(d);
+  float* Qs = lds;                       // [C][QS]
+  float* Ks = Qs + C * QS;               // [C][QS]
+  float* Vs = Ks + C * QS;               // [C][VSS]
+  float* Ps = Vs + C * VSS;              // [C][PSS]
+  float* Ss = Ps + C * PSS;              // [d][VSS]
+  float* n0 = Ss + d * VSS;              // [d]
+  float* ga = n0 + d;                    // [C] a_r
+  float* gM = ga + C;                    // [C] M_j
+  float* gm = gM + C;                    // [C] m_j
+  float* gcoef = gm + C;                 // [C] exp(m_0 - M_j)
+  float* ginv = gcoef + C;               // [C] 1 / den_j
+  float* gw = ginv + C;                  // [C] exp(a_r - M_last)
+
+  const int s = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * VS, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
+  if (t1 <= t0) return;
+  const int slot = slots[s];
+  float* Sg = S_all + ((size_t)slot * H + h) * d * dv;
+  float* ng = n_all + ((size_t)slot * H + h) * d;
+  float m0 = m_all[(size_t)slot * H + h];
+  const float qscale = rsqrtf((float)d);
+  const int oq = h * d, ok = H * d + h * d, ov = 2 * H * d + h * dv + v0;
+  const int oa = 2 * H * d + 2 * H * dv + h, ob = oa + H;
+  const float bi = bias_i[h], bf = bias_f[h];
+
+  for (int i = tid; i < d * VS; i += THREADS) Ss[(i / VS) * VSS + i % VS] = Sg[(size_t)(i / VS) * dv + v0 + i % VS];
+  for (int r = tid; r < d; r += THREADS) n0[r] = ng[r];
+
+  for (int c0 = t0; c0 < t1; c0 += C) {
+    const int len = min(C, t1 - c0);
+    __syncthreads();                                     // the chunk before is done with every buffer
+    // ---- phase 1: rows into LDS, gates
+    for (int i = tid; i < C * (d / 4); i += THREADS) {
+      const int j = i / (d / 4), k = (i % (d / 4)) * 4;
+      float4 q = {0.f, 0.f, 0.f, 0.f}, kk = q;
+      if (j < len) {
+        const float* row = proj + (size_t)(c0 + j) * row_w;
+        q = *reinterpret_cast<const float4*>(row + oq + k);
+        kk = *reinterpret_cast<const float4*>(row + ok + k);
+      }
+      *reinterpret_cast<float4*>(Qs + j * QS + k) = float4{q.x * qscale, q.y * qscale, q.z * qscale, q.w * qscale};
+      *reinterpret_cast<float4*>(Ks + j * QS + k) = kk;
+    }
+    for (int i = tid; i < C * (VS / 4); i += THREADS) {
+      const int j = i / (VS / 4), k = (i % (VS / 4)) * 4;
+      float4 v = {0.f, 0.f, 0.f, 0.f};
+      if (j < len) v = *reinterpret_cast<const float4*>(proj + (size_t)(c0 + j) * row_w + ov + k);
+      *reinterpret_cast<float4*>(Vs + j * VSS + k) = v;
+    }
+    if (wave == 0) {
+      float ig = -INFINITY, fg = 0.f;
+      if (lane < len) {
+        const float* row = proj + (size_t)(c0 + lane) * row_w;
+        const float a = row[oa] + bi, b = row[ob] + bf;
+        ig = cap > 0.f ? cap * tanhf(a / cap) : a;
+        fg = logsigmoid_f(cap > 0.f ? cap * tanhf(b / cap) : b);
+      }
+      float b = fg;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) { const float t = __shfl_up(b, o, 64); if (lane >= o) b += t; }
+      const float a = ig - b;
+      float M = a;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) { const float t = __shfl_up(M, o, 64); if (lane >= o) M = fmaxf(M, t); }
+      M = fmaxf(M, m0);
+      if (lane < C) { ga[lane] = a; gM[lane] = M; gm[lane] = b + M; gcoef[lane] = expf(m0 - M); }
+    }
+    __syncthreads();
+    const float M_last = gM[len - 1], m_last = gm[len - 1];
+    // ---- phase 2: P = (Q K^T) . D on and below the diagonal
+    for (int tile = wave; tile < CT * (CT + 1) / 2; tile += 4) {
+      int ti = 0, rem = tile;
+      while (rem > ti) { rem -= ti + 1; ++ti; }
+      const int tj = rem;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      const float* qa = Qs + (ti * 16 + (lane & 15)) * QS + (lane >> 4);
+      const float* kb = Ks + (tj * 16 + (lane & 15)) * QS + (lane >> 4);
+      for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], kb[kk], acc, 0, 0, 0);
+      const int r = tj * 16 + (lane & 15);
+      const float ar = ga[r];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = ti * 16 + (lane >> 4) * 4 + i;
+        const float w = r <= j ? expf(ar - gM[j]) : 0.f;
+        Ps[j * PSS + r] = acc[i] * w;
+      }
+    }
+    if (tid < C) gw[tid] = tid < len ? expf(ga[tid] - M_last) : 0.f;
+    __syncthreads();
+    // ---- phase 3a: the denominators, four threads a row
+    if (tid < 4 * C) {
+      const int j = tid >> 2, part = tid & 3;
+      float rs = 0.f, nq = 0.f;
+      const int rmax = (j / 16 + 1) * 16;
+      for (int r = part; r < rmax; r += 4) rs += Ps[j * PSS + r];
+      for (int k = part; k < d; k += 4) nq = fmaf(n0[k], Qs[j * QS + k], nq);
+      float tot = fmaf(gcoef[j], nq, rs);
+      tot += __shfl_xor(tot, 1, 64);
+      tot += __shfl_xor(tot, 2, 64);
+      if (part == 0) ginv[j] = 1.f / (fmaxf(fabsf(tot), expf(-gm[j])) + 1e-6f);
+    }
+    __syncthreads();
+    // ---- phase 3b: read-outs (coef . Q S_0 + P V) / den
+    for (int tile = wave; tile < CT * VT; tile += 4) {
+      const int ti = tile / VT, tn = tile % VT;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      const float* qa = Qs + (ti * 16 + (lane & 15)) * QS + (lane >> 4);
+      const float* sb = Ss + (lane >> 4) * VSS + tn * 16 + (lane & 15);
+      for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], sb[kk * VSS], acc, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] *= gcoef[ti * 16 + (lane >> 4) * 4 + i];
+      const float* pa = Ps + (ti * 16 + (lane & 15)) * PSS + (lane >> 4);
+      const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
+      for (int kk = 0; kk < (ti + 1) * 16; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[kk], vb[kk * VSS], acc, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = ti * 16 + (lane >> 4) * 4 + i;
+        if (j < len) work[(size_t)(c0 + j) * H * dv + h * dv + v0 + tn * 16 + (lane & 15)] = acc[i] * ginv[j];
+      }
+    }
+    __syncthreads();                                     // every read of S_0 and n_0 is over
+    // ---- phase 4: the state at the chunk's end
+    const float cS = expf(m0 - M_last);
+    for (int tile = wave; tile < (d / 16) * VT; tile += 4) {
+      const int tk = tile / VT, tn = tile % VT;
+      float* sp = Ss + (tk * 16 + (lane >> 4) * 4) * VSS + tn * 16 + (lane & 15);
+      f32x4_t acc;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = cS * sp[i * VSS];
+      const float* ka = Ks + (lane >> 4) * QS + tk * 16 + (lane & 15);
+      const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
+      for (int kk = 0; kk < C; kk += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kk * QS] * gw[kk + (lane >> 4)], vb[kk * VSS], acc, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sp[i * VSS] = acc[i];
+    }
+    for (int k = tid; k < d; k += THREADS) {
+      float x = cS * n0[k];
+      for (int r = 0; r < len; ++r) x = fmaf(gw[r], Ks[r * QS + k], x);
+      n0[k] = x;
+    }
+    m0 = m_last;
+  }
+  __syncthreads();
+  for (int i = tid; i < d * VS; i += THREADS) Sg[(size_t)(i / VS) * dv + v0 + i % VS] = Ss[(i / VS) * VSS + i % VS];
+  if (blockIdx.z == 0) {
+    for (int r = tid; r < d; r += THREADS) ng[r] = n0[r];
+    if (tid == 0) m_all[(size_t)slot * H + h] = m0;
+  }
+}
+
+// out[t, h, :] = work[t, h, :] / rms(work[t, h, :]) * w[h, :] * sigmoid(g[t, h, :]); a block per (token, head).
+template <typename TO>
+__global__ void mlstm_finish_kernel(const float* __restrict__ work, const float* __restrict__ proj, int row_w,
+                                    const void* __restrict__ norm_w, int norm_dtype, TO* __restrict__ out,
+                                    int H, int d, int dv, float eps) {
+  __shared__ float red[17];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* o = work + (size_t)t * H * dv + h * dv;
+  const float* g = proj + (size_t)t * row_w + 2 * H * d + H * dv + h * dv;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < dv; c += blockDim.x) sq = fmaf(o[c], o[c], sq);
+  sq = block_sum(sq, red);
+  const float inv = 1.f / sqrtf(sq / (float)dv + eps);
+  for (int c = threadIdx.x; c < dv; c += blockDim.x) {
+    const float w = norm_dtype == DT_F32 ? ((const float*)norm_w)[h * dv + c] : bf16_to_f32(((const bf16_t*)norm_w)[h * dv + c]);
+    store_f32(out, (size_t)t * H * dv + h * dv + c, o[c] * inv * w / (1.f + expf(-g[c])));
+  }
+}
+
+size_t chunk_lds_bytes(int C, int VS, int d) {
+  const int QS = d + ((84 - d % 64) % 64), VSS = VS == 32 ? 48 : 80;
+  return (size_t)(2 * C * QS + C * VSS + C * (C + 4) + d * VSS + d + 6 * C) * sizeof(float);
+}
+
+// The chunk length and the columns a block owns for these sizes (0, 0: the chunk kernel does not cover them).
+void chunk_plan(int n_seqs, int H, int d, int dv, int* C, int* VS) {
+  *C = *VS = 0;
+  if (d % 16 || dv % 16 || d > 256) return;
+  const int c = d <= 128 ? 64 : 32;
+  int best = 0;
+  for (int vs = 64; vs >= 16; vs >>= 1) {
+    if (dv % vs || (c == 32 && vs == 64) || chunk_lds_bytes(c, vs, d) > 150 * 1024) continue;
+    if (!best) best = vs;
+    if ((long)n_seqs * H * (dv / best) >= 256) break;      // the widest slice that still makes a block a CU
+    best = vs;
+  }
+  if (best) { *C = c; *VS = best; }
+}
+
 }  // namespace
 
 extern "C" int alice_mlstm_step(const float* proj, int row_w, const float* bias_i, const float* bias_f,
@@ -183,6 +401,58 @@ extern "C" int alice_gelu_mul_rows(const void* z, int z_dtype, const void* table
     else { if (full_precision) GO(bf16_t, bf16_t, true); else GO(bf16_t, bf16_t, false); }
   }
 #undef GO
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int alice_mlstm_chunks_supported(int n_seqs, int H, int d, int dv) {
+  int C, VS;
+  chunk_plan(n_seqs, H, d, dv, &C, &VS);
+  return C != 0;
+}
+
+// The same as alice_mlstm_step for steps of many tokens a sequence, a chunk at a time on the matrix cores;
+// work: float32 [T, H * dv].  Sizes it does not cover (alice_mlstm_chunks_supported) are refused.
+extern "C" int alice_mlstm_chunks(const float* proj, int row_w, const float* bias_i, const float* bias_f,
+                                  const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
+                                  const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
+                                  int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps,
+                                  hipStream_t stream) {
+  ALICE_CHECK(dtype_ok(out_dtype) && dtype_ok(norm_dtype), "mlstm: unknown dtype");
+  ALICE_CHECK(T >= 0 && n_seqs >= 0 && H >= 1 && H <= 65535 && d >= 1 && dv >= 1, "mlstm: bad sizes H=%d d=%d dv=%d", H, d, dv);
+  ALICE_CHECK(row_w >= 2 * H * d + 2 * H * dv + 2 * H && row_w % 4 == 0 && ((uintptr_t)proj & 15) == 0,
+              "mlstm: rows of %d numbers are too short, or not a multiple of four numbers from a 16-byte boundary", row_w);
+  ALICE_CHECK(proj && bias_i && bias_f && norm_w && out && work && cu_seqlens && slots && S && n && m && n_slots >= 1,
+              "mlstm: a pointer is missing");
+  int C, VS;
+  chunk_plan(n_seqs, H, d, dv, &C, &VS);
+  ALICE_CHECK(C != 0, "mlstm: the chunk kernel does not cover head sizes %d and %d", d, dv);
+  if (n_seqs == 0 || T == 0) return 0;
+  const size_t lds = chunk_lds_bytes(C, VS, d);
+  dim3 grid(n_seqs, H, dv / VS);
+#define GO(CC, VV)                                                                                                   \
+  do {                                                                                                               \
+    static bool raised = false; /* blocks of more than 64 KB of shared memory: said once per kernel */              \
+    if (!raised) {                                                                                                   \
+      hipFuncSetAttribute((const void*)mlstm_chunk_kernel<CC, VV>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+      (void)hipGetLastError();                                                                                       \
+      raised = true;                                                                                                 \
+    }                                                                                                                \
+    mlstm_chunk_kernel<CC, VV><<<grid, THREADS, lds, stream>>>(proj, row_w, bias_i, bias_f, work, cu_seqlens, slots, \
+                                                               S, n, m, H, d, dv, cap);                              \
+  } while (0)
+  if (C == 64 && VS == 64) GO(64, 64);
+  else if (C == 64 && VS == 32) GO(64, 32);
+  else if (C == 64) GO(64, 16);
+  else if (VS == 32) GO(32, 32);
+  else GO(32, 16);
+#undef GO
+  ALICE_LAUNCH_CHECK();
+  const int threads = dv >= 256 ? 256 : (dv >= 128 ? 128 : 64);
+  if (out_dtype == DT_F32)
+    mlstm_finish_kernel<float><<<dim3(T, H), threads, 0, stream>>>(work, proj, row_w, norm_w, norm_dtype, (float*)out, H, d, dv, eps);
+  else
+    mlstm_finish_kernel<bf16_t><<<dim3(T, H), threads, 0, stream>>>(work, proj, row_w, norm_w, norm_dtype, (bf16_t*)out, H, d, dv, eps);
   ALICE_LAUNCH_CHECK();
   return 0;
 }

@@ -45,6 +45,8 @@ def _declare(lib) -> None:
         "alice_frag16_supported": [I, I, I],
         "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, I, P],
         "alice_mlstm_step": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, F, F, P],
+        "alice_mlstm_chunks": [P, I, P, P, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
+        "alice_mlstm_chunks_supported": [I, I, I, I],
         "alice_gelu_mul_rows": [P, I, P, I, I, I, P, P, I, I, I, I, I, P],
         "alice_linear_rope_cache": [P, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
@@ -589,9 +591,50 @@ def mlstm(proj, bias_i, bias_f, norm_w, out, ctx, S, n, m, *, heads: int, head_d
 
 def mlstm_rows(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, *, n_seqs: int, max_new: int, heads: int,
                head_dim: int, value_head_dim: int, cap: float, eps: float) -> None:
-    """Picks the kernel for the step's shape: token by token for single tokens and short pieces."""
+    """Picks the kernel for the step's shape: token by token for single tokens and pieces of a few tokens, a chunk
+    of tokens at a time on the matrix cores for longer ones (head sizes that are multiples of 16, keys up to 256)."""
+    if (max_new >= MLSTM_CHUNK_FROM and proj.shape[1] % 4 == 0
+            and library().alice_mlstm_chunks_supported(int(n_seqs), heads, head_dim, value_head_dim)):
+        mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
+                     head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
+        return
     mlstm_step(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
                head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
+
+
+MLSTM_CHUNK_FROM = 4      # steps whose longest piece has at least this many tokens take the chunk kernel
+
+
+def _mlstm_args(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs, H, d, dv):
+    T = proj.shape[0]
+    _dev(proj, "proj", torch.float32)
+    if proj.dim() != 2 or proj.shape[1] < 2 * H * d + 2 * H * dv + 2 * H:
+        raise HipLibraryError(f"proj rows of {tuple(proj.shape)} are too short")
+    _dev(bias_i, "bias_i", torch.float32, (H,))
+    _dev(bias_f, "bias_f", torch.float32, (H,))
+    _dev(norm_w, "norm_w", None, (H * dv,))
+    _dev(out, "out", None, (T, H * dv))
+    _dev(cu_seqlens, "cu_seqlens", torch.int32)
+    _dev(slots, "slots", torch.int32)
+    if cu_seqlens.numel() < n_seqs + 1 or slots.numel() < n_seqs:
+        raise HipLibraryError("cu_seqlens and slots are too short for the step's sequences")
+    n_slots = S.shape[0]
+    _dev(S, "S", torch.float32, (n_slots, H, d, dv))
+    _dev(n, "n", torch.float32, (n_slots, H, d))
+    _dev(m, "m", torch.float32, (n_slots, H))
+    return T, n_slots
+
+
+def mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, *, n_seqs: int, heads: int, head_dim: int,
+                 value_head_dim: int, cap: float, eps: float) -> None:
+    """mlstm_step's result by the chunk kernel (see mlstm.hip); allocates its float32 workspace [T, H dv]."""
+    H, d, dv = heads, head_dim, value_head_dim
+    T, n_slots = _mlstm_args(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs, H, d, dv)
+    work = torch.empty((T, H * dv), dtype=torch.float32, device=proj.device)
+    _call("alice_mlstm_chunks", proj.data_ptr(), proj.shape[1], bias_i.data_ptr(), bias_f.data_ptr(), norm_w.data_ptr(),
+          dtype_code(norm_w.dtype), out.data_ptr(), dtype_code(out.dtype), work.data_ptr(), cu_seqlens.data_ptr(),
+          slots.data_ptr(), S.data_ptr(), n.data_ptr(), m.data_ptr(), T, int(n_seqs), int(n_slots), H, d, dv, float(cap),
+          float(eps), _stream())
 
 
 def mlstm_step(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, norm_w: torch.Tensor, out: torch.Tensor,

@@ -45,7 +45,7 @@ class MatrixMemory(Part):
         self.eps = float(norm_eps)
         self.names = dict(_DEFAULT_NAMES, **(tensor_names or {}))
         self.qk, self.vw = self.nH * self.d, self.nH * self.dv
-        self.row = 2 * self.qk + 2 * self.vw + 2 * self.nH
+        self.row = -(-(2 * self.qk + 2 * self.vw + 2 * self.nH) // 4) * 4      # rows of whole 16-byte units
         self.proj = Linear(hidden_size, self.row, precision)
         self.o = Linear(self.vw, hidden_size, precision)
         self.norm_w: Optional[torch.Tensor] = None
@@ -87,7 +87,10 @@ class MatrixMemory(Part):
         mats = [self.precision.matrix(self._parts.pop(self.names[c])) for c in self._order()]
         if len({m.dtype for m in mats}) > 1:
             mats = [m.float() for m in mats]
-        self.proj.load(torch.cat(mats, dim=0))
+        w = torch.cat(mats, dim=0)
+        if w.shape[0] < self.row:                             # the padding rows: zeros that nobody reads
+            w = torch.cat([w, w.new_zeros(self.row - w.shape[0], w.shape[1])], dim=0)
+        self.proj.load(w)
 
     def weight_bytes(self) -> int:
         return self.proj.nbytes() + self.o.nbytes()

@@ -190,7 +190,7 @@ def novotar_tensors(raw: dict, seed: int):
         elif name in ("embed", "side.embed"):
             t = r * (0.5 if name == "embed" else 1.0)
         else:
-            gain = 3.0 if name.endswith((".i", ".f", "left.q", "left.k", "left.g")) else 1.0
+            gain = 2.0 if name.endswith((".i", ".f", "left.q", "left.k", "left.g")) else 1.0
             t = r * gain / shape[1] ** 0.5
         out[name] = t.to(torch.bfloat16)
     return cfg, out

@@ -47,7 +47,8 @@ def assert_close(got, ref, dtype, what=""):
     such a place is amplified.  The plain implementation itself, run in 32-bit, is within 3e-6 of its 64-bit self
     at the median row and 3e-4 off at the worst rows of these configurations.  32-bit: every logit within 1e-3
     (relative to the largest logit) and the median row within 2e-5.  bfloat16: a row's error is measured as a
-    whole (root mean square against the row's own): the rows' mean within 0.06 and nine rows in ten within 0.1.
+    whole (root mean square against the row's own): the rows' mean within 0.06 and nine rows in ten within 0.1
+    (of twenty rows and more; every row within 0.3 of fewer).
     A wrong key, state or position moves most rows by 0.3 and more."""
     assert got.shape == ref.shape, what
     if dtype == "float32":
@@ -56,7 +57,8 @@ def assert_close(got, ref, dtype, what=""):
         assert float(e.max()) < 1e-3 * scale and float(e.median()) < 2e-5 * scale, (what, float(e.max()), float(e.median()))
     else:
         e = row_errors(got, ref)
-        assert float(e.mean()) < 0.06 and float(e.quantile(0.9)) < 0.1 and float(e.max()) < 1.0, \
+        many = e.numel() >= 20
+        assert float(e.mean()) < 0.06 and float(e.quantile(0.9) if many else e.max()) < (0.1 if many else 0.3) and float(e.max()) < 1.0, \
             (what, float(e.max()), float(e.mean()))
 
 
