@@ -99,6 +99,8 @@ int alice_attention_prefill(const void* q, const void* k_pool, const void* v_poo
                             const int* cu_seqlens, const int* context_lens, const int* block_table,
                             int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
                             float scale, float softcap, int window, int variant, int out_layout, hipStream_t stream);
+// out[t, h, :] *= sigmoid(gate[t * gate_stride + h]) in place on a bfloat16 attention output in either layout.
+int alice_head_gate(void* out, int out_layout, const void* gate, int gate_stride, int T, int nH, int d, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 // out may be absent when splits > 1: the splits are then left in `parts`, [B][nH][splits][ALICE_ATTN_PARTS_HEAD + d]
 // = (maximum as a base-2 exponent, sum, two unused, unnormalised output: the output starts at a multiple of 16
@@ -126,8 +128,14 @@ int alice_mlstm_step(const float* proj, int row_w, const float* bias_i, const fl
                      const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
                      int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, hipStream_t stream);
 
+// alice_mlstm_cols: the same result for single tokens and pieces of a few, key sizes up to 256: a block per
+// (sequence, head, 64 value columns), the state in registers, read and written once a step.
 // The same for steps of many tokens a sequence, a chunk of tokens at a time on the 32-bit matrix instruction;
-// work: float32 [T, H * dv].  alice_mlstm_chunks_supported says whether the head sizes are covered.
+// work: T * (H * dv + H) float32 (alice_mlstm_cols: T * H * dv).  alice_mlstm_chunks_supported says whether the head sizes are covered.
+int alice_mlstm_cols(const float* proj, int row_w, const float* bias_i, const float* bias_f,
+                     const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
+                     const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
+                     int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, hipStream_t stream);
 int alice_mlstm_chunks_supported(int n_seqs, int H, int d, int dv);
 int alice_mlstm_chunks(const float* proj, int row_w, const float* bias_i, const float* bias_f,
                        const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,

@@ -722,6 +722,37 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_
 // Head sizes the matrix-core kernels and the fragment cache layout cover.
 extern "C" int alice_attention_mfma_supported(int d) { return d == 64 || d == 128 || d == 256; }
 
+namespace {
+// out[t, h, :] *= sigmoid(gate[t * gate_stride + h]) in place, in either output layout; eight elements a thread.
+__global__ void head_gate_kernel(bf16_t* __restrict__ out, int out_layout, const bf16_t* __restrict__ gate, int gate_stride,
+                                 int T, int nH, int D) {
+  const int per_row = nH * D / 8;
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (size_t)T * per_row) return;
+  const int t = (int)(i / per_row), c = (int)(i % per_row) * 8;
+  const float s = 1.f / (1.f + __expf(-bf16_to_f32(gate[(size_t)t * gate_stride + c / D])));
+  uint4* p = reinterpret_cast<uint4*>(out + decode_out_index(out_layout, t, c, nH * D));
+  uint4 v = *p;
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) w[k] = pack_bf16x2(bf16_bits_to_f32(w[k] & 0xffffu) * s, bf16_bits_to_f32(w[k] >> 16) * s);
+  *p = uint4{w[0], w[1], w[2], w[3]};
+}
+}  // namespace
+
+// One gate number a head: out[t, h, :] *= sigmoid(gate[t * gate_stride + h]), in place, on the output of the
+// matrix-core attention kernels in either layout (bfloat16, head size a multiple of 8).
+extern "C" int alice_head_gate(void* out, int out_layout, const void* gate, int gate_stride, int T, int nH, int d,
+                               hipStream_t stream) {
+  ALICE_CHECK(out && gate && T >= 0 && nH >= 1 && d >= 8 && d % 8 == 0 && gate_stride >= nH, "head_gate: bad sizes T=%d nH=%d d=%d", T, nH, d);
+  ALICE_CHECK(out_layout == 0 || (out_layout == 1 && (nH * d) % 32 == 0), "head_gate: unknown output layout %d", out_layout);
+  if (T == 0) return 0;
+  const size_t n = (size_t)T * (nH * d / 8);
+  head_gate_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((bf16_t*)out, out_layout, (const bf16_t*)gate, gate_stride, T, nH, d);
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int alice_attention_prefill(const void* q, const void* k_pool, const void* v_pool, void* out,
                                        const int* cu_seqlens, const int* context_lens, const int* block_table,
                                        int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,

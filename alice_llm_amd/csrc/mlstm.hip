@@ -152,10 +152,13 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int lds_pad20(int d) { return d + ((84 - d % 64) % 64); }   // stride = 20 mod 64 banks
 
+constexpr int CTHREADS = 512;     // eight waves a block: two a SIMD, so that one's LDS reads hide behind the other's products
+constexpr int CWAVES = CTHREADS / 64;
+
 template <int C, int VS>
-__global__ __launch_bounds__(THREADS) void mlstm_chunk_kernel(
+__global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
     const float* __restrict__ proj, int row_w, const float* __restrict__ bias_i, const float* __restrict__ bias_f,
-    float* __restrict__ work, const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
+    float* __restrict__ work, float* __restrict__ dens, const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
     float* __restrict__ S_all, float* __restrict__ n_all, float* __restrict__ m_all,
     int H, int d, int dv, float cap) {
   constexpr int VSS = VS == 32 ? 48 : 80;      // row stride of V and S tiles: 16 mod 64 banks
@@ -173,8 +176,7 @@ __global__ __launch_bounds__(THREADS) void mlstm_chunk_kernel(
   float* gM = ga + C;                    // [C] M_j
   float* gm = gM + C;                    // [C] m_j
   float* gcoef = gm + C;                 // [C] exp(m_0 - M_j)
-  float* ginv = gcoef + C;               // [C] 1 / den_j
-  float* gw = ginv + C;                  // [C] exp(a_r - M_last)
+  float* gw = gcoef + C;                 // [C] exp(a_r - M_last)
 
   const int s = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * VS, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -189,58 +191,95 @@ __global__ __launch_bounds__(THREADS) void mlstm_chunk_kernel(
   const int oa = 2 * H * d + 2 * H * dv + h, ob = oa + H;
   const float bi = bias_i[h], bf = bias_f[h];
 
-  for (int i = tid; i < d * VS; i += THREADS) Ss[(i / VS) * VSS + i % VS] = Sg[(size_t)(i / VS) * dv + v0 + i % VS];
-  for (int r = tid; r < d; r += THREADS) n0[r] = ng[r];
+  for (int i = tid; i < d * VS; i += CTHREADS) Ss[(i / VS) * VSS + i % VS] = Sg[(size_t)(i / VS) * dv + v0 + i % VS];
+  for (int r = tid; r < d; r += CTHREADS) n0[r] = ng[r];
+
+  // A chunk's rows are fetched into registers while the chunk before is worked on, and its gates' tanh and
+  // logarithm are taken by wave 0 at the end of that chunk: neither waits in a chunk's own time.
+  constexpr int NQ = 4, NV = 2;                          // float4s a thread fetches at most (checked by the host's plan)
+  const int q4 = C * (d / 4);
+  float4 rq[NQ], rk[NQ], rv[NV];
+  float raw_a = 0.f, raw_b = 0.f, ig_n = -INFINITY, fg_n = 0.f;
+  auto fetch = [&](int c0) {
+    const int len = min(C, t1 - c0);
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+      const int i = tid + u * CTHREADS;
+      const int j = i / (d / 4), k = (i % (d / 4)) * 4;
+      rq[u] = rk[u] = float4{0.f, 0.f, 0.f, 0.f};
+      if (i < q4 && j < len) {
+        const float* row = proj + (size_t)(c0 + j) * row_w;
+        rq[u] = *reinterpret_cast<const float4*>(row + oq + k);
+        rk[u] = *reinterpret_cast<const float4*>(row + ok + k);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int i = tid + u * CTHREADS;
+      const int j = i / (VS / 4), k = (i % (VS / 4)) * 4;
+      rv[u] = float4{0.f, 0.f, 0.f, 0.f};
+      if (i < C * (VS / 4) && j < len) rv[u] = *reinterpret_cast<const float4*>(proj + (size_t)(c0 + j) * row_w + ov + k);
+    }
+    if (wave == 0 && lane < len) {
+      const float* row = proj + (size_t)(c0 + lane) * row_w;
+      raw_a = row[oa];
+      raw_b = row[ob];
+    }
+  };
+  auto gates_ahead = [&](int c0) {                       // wave 0: the log gates of the fetched chunk
+    ig_n = -INFINITY;
+    fg_n = 0.f;
+    if (lane < min(C, t1 - c0)) {
+      const float a = raw_a + bi, b = raw_b + bf;
+      ig_n = cap > 0.f ? cap * tanhf(a / cap) : a;
+      fg_n = logsigmoid_f(cap > 0.f ? cap * tanhf(b / cap) : b);
+    }
+  };
+  fetch(t0);
+  if (wave == 0) gates_ahead(t0);
 
   for (int c0 = t0; c0 < t1; c0 += C) {
     const int len = min(C, t1 - c0);
     __syncthreads();                                     // the chunk before is done with every buffer
-    // ---- phase 1: rows into LDS, gates
-    for (int i = tid; i < C * (d / 4); i += THREADS) {
-      const int j = i / (d / 4), k = (i % (d / 4)) * 4;
-      float4 q = {0.f, 0.f, 0.f, 0.f}, kk = q;
-      if (j < len) {
-        const float* row = proj + (size_t)(c0 + j) * row_w;
-        q = *reinterpret_cast<const float4*>(row + oq + k);
-        kk = *reinterpret_cast<const float4*>(row + ok + k);
+    // ---- phase 1: the fetched rows into LDS, the gates' running sums and maxima
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+      const int i = tid + u * CTHREADS;
+      if (i < q4) {
+        const int j = i / (d / 4), k = (i % (d / 4)) * 4;
+        *reinterpret_cast<float4*>(Qs + j * QS + k) = float4{rq[u].x * qscale, rq[u].y * qscale, rq[u].z * qscale, rq[u].w * qscale};
+        *reinterpret_cast<float4*>(Ks + j * QS + k) = rk[u];
       }
-      *reinterpret_cast<float4*>(Qs + j * QS + k) = float4{q.x * qscale, q.y * qscale, q.z * qscale, q.w * qscale};
-      *reinterpret_cast<float4*>(Ks + j * QS + k) = kk;
     }
-    for (int i = tid; i < C * (VS / 4); i += THREADS) {
-      const int j = i / (VS / 4), k = (i % (VS / 4)) * 4;
-      float4 v = {0.f, 0.f, 0.f, 0.f};
-      if (j < len) v = *reinterpret_cast<const float4*>(proj + (size_t)(c0 + j) * row_w + ov + k);
-      *reinterpret_cast<float4*>(Vs + j * VSS + k) = v;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int i = tid + u * CTHREADS;
+      if (i < C * (VS / 4)) *reinterpret_cast<float4*>(Vs + (i / (VS / 4)) * VSS + (i % (VS / 4)) * 4) = rv[u];
     }
     if (wave == 0) {
-      float ig = -INFINITY, fg = 0.f;
-      if (lane < len) {
-        const float* row = proj + (size_t)(c0 + lane) * row_w;
-        const float a = row[oa] + bi, b = row[ob] + bf;
-        ig = cap > 0.f ? cap * tanhf(a / cap) : a;
-        fg = logsigmoid_f(cap > 0.f ? cap * tanhf(b / cap) : b);
-      }
-      float b = fg;
+      float b = fg_n;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) { const float t = __shfl_up(b, o, 64); if (lane >= o) b += t; }
-      const float a = ig - b;
+      const float a = ig_n - b;
       float M = a;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) { const float t = __shfl_up(M, o, 64); if (lane >= o) M = fmaxf(M, t); }
       M = fmaxf(M, m0);
       if (lane < C) { ga[lane] = a; gM[lane] = M; gm[lane] = b + M; gcoef[lane] = expf(m0 - M); }
     }
+    const bool more = c0 + C < t1;
+    if (more) fetch(c0 + C);
     __syncthreads();
     const float M_last = gM[len - 1], m_last = gm[len - 1];
     // ---- phase 2: P = (Q K^T) . D on and below the diagonal
-    for (int tile = wave; tile < CT * (CT + 1) / 2; tile += 4) {
+    for (int tile = wave; tile < CT * (CT + 1) / 2; tile += CWAVES) {
       int ti = 0, rem = tile;
       while (rem > ti) { rem -= ti + 1; ++ti; }
       const int tj = rem;
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
       const float* qa = Qs + (ti * 16 + (lane & 15)) * QS + (lane >> 4);
       const float* kb = Ks + (tj * 16 + (lane & 15)) * QS + (lane >> 4);
+#pragma unroll 8
       for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], kb[kk], acc, 0, 0, 0);
       const int r = tj * 16 + (lane & 15);
       const float ar = ga[r];
@@ -253,90 +292,197 @@ __global__ __launch_bounds__(THREADS) void mlstm_chunk_kernel(
     }
     if (tid < C) gw[tid] = tid < len ? expf(ga[tid] - M_last) : 0.f;
     __syncthreads();
-    // ---- phase 3a: the denominators, four threads a row
-    if (tid < 4 * C) {
-      const int j = tid >> 2, part = tid & 3;
-      float rs = 0.f, nq = 0.f;
-      const int rmax = (j / 16 + 1) * 16;
-      for (int r = part; r < rmax; r += 4) rs += Ps[j * PSS + r];
-      for (int k = part; k < d; k += 4) nq = fmaf(n0[k], Qs[j * QS + k], nq);
-      float tot = fmaf(gcoef[j], nq, rs);
-      tot += __shfl_xor(tot, 1, 64);
-      tot += __shfl_xor(tot, 2, 64);
-      if (part == 0) ginv[j] = 1.f / (fmaxf(fabsf(tot), expf(-gm[j])) + 1e-6f);
-    }
-    __syncthreads();
-    // ---- phase 3b: read-outs (coef . Q S_0 + P V) / den
-    for (int tile = wave; tile < CT * VT; tile += 4) {
-      const int ti = tile / VT, tn = tile % VT;
+    // ---- phase 3: read-outs coef . Q S_0 + P V, unnormalised; the blocks of a head's first columns also take
+    // n . q the same way (n as one more column: Q n_0 and the row sums of P) and leave the denominators
+    const int n_tiles3 = CT * VT + (blockIdx.z == 0 ? CT : 0);
+    for (int tile = wave; tile < n_tiles3; tile += CWAVES) {
+      const bool is_n = tile >= CT * VT;
+      const int ti = is_n ? tile - CT * VT : tile / VT, tn = is_n ? 0 : tile % VT;
+      const bool col0 = (lane & 15) == 0;
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
       const float* qa = Qs + (ti * 16 + (lane & 15)) * QS + (lane >> 4);
-      const float* sb = Ss + (lane >> 4) * VSS + tn * 16 + (lane & 15);
-      for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], sb[kk * VSS], acc, 0, 0, 0);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[i] *= gcoef[ti * 16 + (lane >> 4) * 4 + i];
       const float* pa = Ps + (ti * 16 + (lane & 15)) * PSS + (lane >> 4);
-      const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
-      for (int kk = 0; kk < (ti + 1) * 16; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[kk], vb[kk * VSS], acc, 0, 0, 0);
+      if (!is_n) {
+        const float* sb = Ss + (lane >> 4) * VSS + tn * 16 + (lane & 15);
+#pragma unroll 8
+        for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], sb[kk * VSS], acc, 0, 0, 0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = ti * 16 + (lane >> 4) * 4 + i;
-        if (j < len) work[(size_t)(c0 + j) * H * dv + h * dv + v0 + tn * 16 + (lane & 15)] = acc[i] * ginv[j];
+        for (int i = 0; i < 4; ++i) acc[i] *= gcoef[ti * 16 + (lane >> 4) * 4 + i];
+        const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
+#pragma unroll 4
+        for (int kk = 0; kk < (ti + 1) * 16; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[kk], vb[kk * VSS], acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = ti * 16 + (lane >> 4) * 4 + i;
+          if (j < len) work[(size_t)(c0 + j) * H * dv + h * dv + v0 + tn * 16 + (lane & 15)] = acc[i];
+        }
+      } else {
+        const float* nb = n0 + (lane >> 4);
+#pragma unroll 8
+        for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], col0 ? nb[kk] : 0.f, acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= gcoef[ti * 16 + (lane >> 4) * 4 + i];
+        const float one = col0 ? 1.f : 0.f;
+#pragma unroll 4
+        for (int kk = 0; kk < (ti + 1) * 16; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[kk], one, acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = ti * 16 + (lane >> 4) * 4 + i;
+          if (col0 && j < len) dens[(size_t)(c0 + j) * H + h] = fmaxf(fabsf(acc[i]), expf(-gm[j])) + 1e-6f;
+        }
       }
     }
     __syncthreads();                                     // every read of S_0 and n_0 is over
-    // ---- phase 4: the state at the chunk's end
+    // ---- phase 4: the state at the chunk's end (n again as one more column)
     const float cS = expf(m0 - M_last);
-    for (int tile = wave; tile < (d / 16) * VT; tile += 4) {
-      const int tk = tile / VT, tn = tile % VT;
-      float* sp = Ss + (tk * 16 + (lane >> 4) * 4) * VSS + tn * 16 + (lane & 15);
-      f32x4_t acc;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[i] = cS * sp[i * VSS];
+    const int n_tiles4 = (d / 16) * VT + (blockIdx.z == 0 ? d / 16 : 0);
+    for (int tile = wave; tile < n_tiles4; tile += CWAVES) {
+      const bool is_n = tile >= (d / 16) * VT;
+      const int tk = is_n ? tile - (d / 16) * VT : tile / VT, tn = is_n ? 0 : tile % VT;
+      const bool col0 = (lane & 15) == 0;
       const float* ka = Ks + (lane >> 4) * QS + tk * 16 + (lane & 15);
-      const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
-      for (int kk = 0; kk < C; kk += 4)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kk * QS] * gw[kk + (lane >> 4)], vb[kk * VSS], acc, 0, 0, 0);
+      f32x4_t acc;
+      if (!is_n) {
+        float* sp = Ss + (tk * 16 + (lane >> 4) * 4) * VSS + tn * 16 + (lane & 15);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sp[i * VSS] = acc[i];
-    }
-    for (int k = tid; k < d; k += THREADS) {
-      float x = cS * n0[k];
-      for (int r = 0; r < len; ++r) x = fmaf(gw[r], Ks[r * QS + k], x);
-      n0[k] = x;
+        for (int i = 0; i < 4; ++i) acc[i] = cS * sp[i * VSS];
+        const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
+#pragma unroll 8
+        for (int kk = 0; kk < C; kk += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kk * QS] * gw[kk + (lane >> 4)], vb[kk * VSS], acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sp[i * VSS] = acc[i];
+      } else {
+        float* np = n0 + tk * 16 + (lane >> 4) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = col0 ? cS * np[i] : 0.f;
+        const float one = col0 ? 1.f : 0.f;
+#pragma unroll 8
+        for (int kk = 0; kk < C; kk += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kk * QS] * gw[kk + (lane >> 4)], one, acc, 0, 0, 0);
+        if (col0) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) np[i] = acc[i];
+        }
+      }
     }
     m0 = m_last;
+    if (more && wave == 0) gates_ahead(c0 + C);
   }
   __syncthreads();
-  for (int i = tid; i < d * VS; i += THREADS) Sg[(size_t)(i / VS) * dv + v0 + i % VS] = Ss[(i / VS) * VSS + i % VS];
+  for (int i = tid; i < d * VS; i += CTHREADS) Sg[(size_t)(i / VS) * dv + v0 + i % VS] = Ss[(i / VS) * VSS + i % VS];
   if (blockIdx.z == 0) {
-    for (int r = tid; r < d; r += THREADS) ng[r] = n0[r];
+    for (int r = tid; r < d; r += CTHREADS) ng[r] = n0[r];
     if (tid == 0) m_all[(size_t)slot * H + h] = m0;
   }
 }
 
-// out[t, h, :] = work[t, h, :] / rms(work[t, h, :]) * w[h, :] * sigmoid(g[t, h, :]); a block per (token, head).
+
+// Single tokens (and pieces of a few): a block per (sequence, head, 64 value columns).  Lane l of every wave owns
+// column c = 64 z + l; wave w owns the rows r = w, w + 4, ...; a thread keeps its RPT elements of S in registers
+// over the sequence's tokens, so the state is read once and written once, in 256-byte runs.  The head norm needs
+// every column: the read-outs go to the 32-bit workspace and mlstm_finish_kernel does the rest.
+template <int RPT>
+__global__ __launch_bounds__(THREADS) void mlstm_cols_kernel(
+    const float* __restrict__ proj, int row_w, const float* __restrict__ bias_i, const float* __restrict__ bias_f,
+    float* __restrict__ work, const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
+    float* __restrict__ S_all, float* __restrict__ n_all, float* __restrict__ m_all,
+    int H, int d, int dv, float cap) {
+  extern __shared__ float lds[];
+  float* qs = lds;                 // d
+  float* ks = qs + d;              // d
+  float* ns = ks + d;              // d
+  float* part = ns + d;            // 4 * 64
+  __shared__ float red[17];
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c = blockIdx.z * 64 + lane;
+  const bool col = c < dv;
+  const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
+  if (t1 <= t0) return;
+  const int slot = slots[s];
+  float* S = S_all + ((size_t)slot * H + h) * d * dv;
+  float* ng = n_all + ((size_t)slot * H + h) * d;
+  float m = m_all[(size_t)slot * H + h];
+  float st[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    const int r = w + 4 * i;
+    st[i] = (col && r < d) ? S[(size_t)r * dv + c] : 0.f;
+  }
+  for (int r = tid; r < d; r += THREADS) ns[r] = ng[r];
+  const float qscale = rsqrtf((float)d);
+  const int oq = h * d, ok = H * d + h * d, ov = 2 * H * d + h * dv;
+  const int oa = 2 * H * d + 2 * H * dv + h, ob = oa + H;
+  const float bi = bias_i[h], bf = bias_f[h];
+  for (int t = t0; t < t1; ++t) {
+    const float* row = proj + (size_t)t * row_w;
+    __syncthreads();
+    for (int r = tid; r < d; r += THREADS) { qs[r] = row[oq + r] * qscale; ks[r] = row[ok + r]; }
+    const float v = col ? row[ov + c] : 0.f;
+    const GateNumbers gn = gate_numbers(row[oa] + bi, row[ob] + bf, cap, m);
+    __syncthreads();
+    float nq = 0.f;
+    for (int r = tid; r < d; r += THREADS) {
+      const float x = fmaf(gn.keep, ns[r], gn.put * ks[r]);
+      ns[r] = x;
+      nq = fmaf(x, qs[r], nq);
+    }
+    nq = block_sum(nq, red);
+    const float pv = gn.put * v;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      const int r = w + 4 * i;
+      if (r < d) {
+        st[i] = fmaf(gn.keep, st[i], ks[r] * pv);
+        acc = fmaf(st[i], qs[r], acc);
+      }
+    }
+    part[w * 64 + lane] = acc;
+    __syncthreads();
+    if (w == 0 && col) {
+      const float den = fmaxf(fabsf(nq), expf(-gn.m_new)) + 1e-6f;
+      work[(size_t)t * H * dv + h * dv + c] = (part[lane] + part[64 + lane] + part[128 + lane] + part[192 + lane]) / den;
+    }
+    m = gn.m_new;
+  }
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    const int r = w + 4 * i;
+    if (col && r < d) S[(size_t)r * dv + c] = st[i];
+  }
+  if (blockIdx.z == 0) {
+    __syncthreads();
+    for (int r = tid; r < d; r += THREADS) ng[r] = ns[r];
+    if (tid == 0) m_all[(size_t)slot * H + h] = m;
+  }
+}
+
+// With o = work[t, h, :] (divided by dens[t, h] where the read-outs were left unnormalised):
+// out[t, h, :] = o / rms(o) * w[h, :] * sigmoid(g[t, h, :]); a block per (token, head).
 template <typename TO>
-__global__ void mlstm_finish_kernel(const float* __restrict__ work, const float* __restrict__ proj, int row_w,
+__global__ void mlstm_finish_kernel(const float* __restrict__ work, const float* __restrict__ dens,
+                                    const float* __restrict__ proj, int row_w,
                                     const void* __restrict__ norm_w, int norm_dtype, TO* __restrict__ out,
                                     int H, int d, int dv, float eps) {
   __shared__ float red[17];
   const int t = blockIdx.x, h = blockIdx.y;
   const float* o = work + (size_t)t * H * dv + h * dv;
   const float* g = proj + (size_t)t * row_w + 2 * H * d + H * dv + h * dv;
+  const float den = dens ? dens[(size_t)t * H + h] : 1.f;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < dv; c += blockDim.x) sq = fmaf(o[c], o[c], sq);
+  for (int c = threadIdx.x; c < dv; c += blockDim.x) { const float x = o[c] / den; sq = fmaf(x, x, sq); }
   sq = block_sum(sq, red);
   const float inv = 1.f / sqrtf(sq / (float)dv + eps);
   for (int c = threadIdx.x; c < dv; c += blockDim.x) {
     const float w = norm_dtype == DT_F32 ? ((const float*)norm_w)[h * dv + c] : bf16_to_f32(((const bf16_t*)norm_w)[h * dv + c]);
-    store_f32(out, (size_t)t * H * dv + h * dv + c, o[c] * inv * w / (1.f + expf(-g[c])));
+    store_f32(out, (size_t)t * H * dv + h * dv + c, o[c] / den * inv * w / (1.f + expf(-g[c])));
   }
 }
 
 size_t chunk_lds_bytes(int C, int VS, int d) {
   const int QS = d + ((84 - d % 64) % 64), VSS = VS == 32 ? 48 : 80;
-  return (size_t)(2 * C * QS + C * VSS + C * (C + 4) + d * VSS + d + 6 * C) * sizeof(float);
+  return (size_t)(2 * C * QS + C * VSS + C * (C + 4) + d * VSS + d + 5 * C) * sizeof(float);
 }
 
 // The chunk length and the columns a block owns for these sizes (0, 0: the chunk kernel does not cover them).
@@ -347,6 +493,7 @@ void chunk_plan(int n_seqs, int H, int d, int dv, int* C, int* VS) {
   int best = 0;
   for (int vs = 64; vs >= 16; vs >>= 1) {
     if (dv % vs || (c == 32 && vs == 64) || chunk_lds_bytes(c, vs, d) > 150 * 1024) continue;
+    if (c * (d / 4) > 4 * CTHREADS || c * (vs / 4) > 2 * CTHREADS) continue;        // what a thread fetches ahead
     if (!best) best = vs;
     if ((long)n_seqs * H * (dv / best) >= 256) break;      // the widest slice that still makes a block a CU
     best = vs;
@@ -405,6 +552,37 @@ extern "C" int alice_gelu_mul_rows(const void* z, int z_dtype, const void* table
   return 0;
 }
 
+// alice_mlstm_step's result for key sizes up to 256 with the state read and written once a step, in blocks of 64
+// value columns; work: float32 [T, H * dv].
+extern "C" int alice_mlstm_cols(const float* proj, int row_w, const float* bias_i, const float* bias_f,
+                                const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
+                                const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
+                                int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps,
+                                hipStream_t stream) {
+  ALICE_CHECK(dtype_ok(out_dtype) && dtype_ok(norm_dtype), "mlstm: unknown dtype");
+  ALICE_CHECK(T >= 0 && n_seqs >= 0 && H >= 1 && H <= 65535 && d >= 1 && d <= 256 && dv >= 1 && dv <= 64 * 65535,
+              "mlstm: bad sizes H=%d d=%d dv=%d (keys up to 256 here)", H, d, dv);
+  ALICE_CHECK(row_w >= 2 * H * d + 2 * H * dv + 2 * H, "mlstm: rows of %d numbers are too short", row_w);
+  ALICE_CHECK(proj && bias_i && bias_f && norm_w && out && work && cu_seqlens && slots && S && n && m && n_slots >= 1,
+              "mlstm: a pointer is missing");
+  if (n_seqs == 0 || T == 0) return 0;
+  dim3 grid(n_seqs, H, (dv + 63) / 64);
+  const size_t lds = (size_t)(3 * d + 256) * sizeof(float);
+#define GO(R) mlstm_cols_kernel<R><<<grid, THREADS, lds, stream>>>(proj, row_w, bias_i, bias_f, work, cu_seqlens, slots, S, n, m, H, d, dv, cap)
+  if (d <= 64) GO(16);
+  else if (d <= 128) GO(32);
+  else GO(64);
+#undef GO
+  ALICE_LAUNCH_CHECK();
+  const int threads = dv >= 256 ? 256 : (dv >= 128 ? 128 : 64);
+  if (out_dtype == DT_F32)
+    mlstm_finish_kernel<float><<<dim3(T, H), threads, 0, stream>>>(work, nullptr, proj, row_w, norm_w, norm_dtype, (float*)out, H, d, dv, eps);
+  else
+    mlstm_finish_kernel<bf16_t><<<dim3(T, H), threads, 0, stream>>>(work, nullptr, proj, row_w, norm_w, norm_dtype, (bf16_t*)out, H, d, dv, eps);
+  ALICE_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int alice_mlstm_chunks_supported(int n_seqs, int H, int d, int dv) {
   int C, VS;
   chunk_plan(n_seqs, H, d, dv, &C, &VS);
@@ -412,7 +590,7 @@ extern "C" int alice_mlstm_chunks_supported(int n_seqs, int H, int d, int dv) {
 }
 
 // The same as alice_mlstm_step for steps of many tokens a sequence, a chunk at a time on the matrix cores;
-// work: float32 [T, H * dv].  Sizes it does not cover (alice_mlstm_chunks_supported) are refused.
+// work: T * (H * dv + H) float32.  Sizes it does not cover (alice_mlstm_chunks_supported) are refused.
 extern "C" int alice_mlstm_chunks(const float* proj, int row_w, const float* bias_i, const float* bias_f,
                                   const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
                                   const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
@@ -429,6 +607,7 @@ extern "C" int alice_mlstm_chunks(const float* proj, int row_w, const float* bia
   ALICE_CHECK(C != 0, "mlstm: the chunk kernel does not cover head sizes %d and %d", d, dv);
   if (n_seqs == 0 || T == 0) return 0;
   const size_t lds = chunk_lds_bytes(C, VS, d);
+  float* dens = work + (size_t)T * H * dv;               // the denominators, [T, H], behind the read-outs
   dim3 grid(n_seqs, H, dv / VS);
 #define GO(CC, VV)                                                                                                   \
   do {                                                                                                               \
@@ -438,7 +617,7 @@ extern "C" int alice_mlstm_chunks(const float* proj, int row_w, const float* bia
       (void)hipGetLastError();                                                                                       \
       raised = true;                                                                                                 \
     }                                                                                                                \
-    mlstm_chunk_kernel<CC, VV><<<grid, THREADS, lds, stream>>>(proj, row_w, bias_i, bias_f, work, cu_seqlens, slots, \
+    mlstm_chunk_kernel<CC, VV><<<grid, CTHREADS, lds, stream>>>(proj, row_w, bias_i, bias_f, work, dens, cu_seqlens, slots, \
                                                                S, n, m, H, d, dv, cap);                              \
   } while (0)
   if (C == 64 && VS == 64) GO(64, 64);
@@ -450,9 +629,9 @@ extern "C" int alice_mlstm_chunks(const float* proj, int row_w, const float* bia
   ALICE_LAUNCH_CHECK();
   const int threads = dv >= 256 ? 256 : (dv >= 128 ? 128 : 64);
   if (out_dtype == DT_F32)
-    mlstm_finish_kernel<float><<<dim3(T, H), threads, 0, stream>>>(work, proj, row_w, norm_w, norm_dtype, (float*)out, H, d, dv, eps);
+    mlstm_finish_kernel<float><<<dim3(T, H), threads, 0, stream>>>(work, dens, proj, row_w, norm_w, norm_dtype, (float*)out, H, d, dv, eps);
   else
-    mlstm_finish_kernel<bf16_t><<<dim3(T, H), threads, 0, stream>>>(work, proj, row_w, norm_w, norm_dtype, (bf16_t*)out, H, d, dv, eps);
+    mlstm_finish_kernel<bf16_t><<<dim3(T, H), threads, 0, stream>>>(work, dens, proj, row_w, norm_w, norm_dtype, (bf16_t*)out, H, d, dv, eps);
   ALICE_LAUNCH_CHECK();
   return 0;
 }

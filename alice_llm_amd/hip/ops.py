@@ -47,12 +47,14 @@ def _declare(lib) -> None:
         "alice_mlstm_step": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, F, F, P],
         "alice_mlstm_chunks": [P, I, P, P, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
         "alice_mlstm_chunks_supported": [I, I, I, I],
+        "alice_mlstm_cols": [P, I, P, P, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
         "alice_gelu_mul_rows": [P, I, P, I, I, I, P, P, I, I, I, I, I, P],
         "alice_linear_rope_cache": [P, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, P],
+        "alice_head_gate": [P, I, P, I, I, I, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
@@ -559,18 +561,20 @@ def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: 
     host-side sizes of the step.  out_layout FRAG16 is taken by the matrix-core kernels only; a score bias
     (bias_slopes, see attention_generic) by the generic kernel only, over a row-major cache."""
     if kv_layout == KV_FRAGMENT:
-        if bias_slopes is not None or gate is not None:
-            raise HipLibraryError("the matrix-core attention kernels take no score bias and no gate: lay the cache out row-major")
+        if bias_slopes is not None:
+            raise HipLibraryError("the matrix-core attention kernels take no score bias: lay the cache out row-major")
         nKV = k_pool.shape[1]
         if ctx.is_decode and num_heads // nKV <= 16:
             attention_decode(q, k_pool, v_pool, out, ctx.context_lens, block_table, num_heads=num_heads,
                              max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
                              out_layout=out_layout)
-            return
-        attention_prefill(q, k_pool, v_pool, out, ctx.cu_seqlens, ctx.context_lens, block_table,
-                          num_heads=num_heads, n_seqs=ctx.n_seqs, max_new=ctx.max_new,
-                          max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
-                          out_layout=out_layout)
+        else:
+            attention_prefill(q, k_pool, v_pool, out, ctx.cu_seqlens, ctx.context_lens, block_table,
+                              num_heads=num_heads, n_seqs=ctx.n_seqs, max_new=ctx.max_new,
+                              max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
+                              out_layout=out_layout)
+        if gate is not None:
+            head_gate(out, out_layout, gate, q.shape[0], num_heads, k_pool.shape[3])
         return
     if out_layout != LAYOUT_ROW:
         raise HipLibraryError("only the matrix-core attention kernels write fragment order")
@@ -598,10 +602,15 @@ def mlstm_rows(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, *,
         mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
                      head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
         return
+    if head_dim <= MLSTM_COLS_MAX_KEY_DIM:
+        mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
+                     head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps, entry="alice_mlstm_cols")
+        return
     mlstm_step(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
                head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
 
 
+MLSTM_COLS_MAX_KEY_DIM = 256      # key sizes up to this keep the state in registers over a step (alice_mlstm_cols)
 MLSTM_CHUNK_FROM = 4      # steps whose longest piece has at least this many tokens take the chunk kernel
 
 
@@ -626,12 +635,13 @@ def _mlstm_args(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n
 
 
 def mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, *, n_seqs: int, heads: int, head_dim: int,
-                 value_head_dim: int, cap: float, eps: float) -> None:
-    """mlstm_step's result by the chunk kernel (see mlstm.hip); allocates its float32 workspace [T, H dv]."""
+                 value_head_dim: int, cap: float, eps: float, entry: str = "alice_mlstm_chunks") -> None:
+    """mlstm_step's result by the chunk kernel, or with entry="alice_mlstm_cols" by the kernel of single tokens
+    (see mlstm.hip); allocates their float32 workspace [T, H dv]."""
     H, d, dv = heads, head_dim, value_head_dim
     T, n_slots = _mlstm_args(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs, H, d, dv)
-    work = torch.empty((T, H * dv), dtype=torch.float32, device=proj.device)
-    _call("alice_mlstm_chunks", proj.data_ptr(), proj.shape[1], bias_i.data_ptr(), bias_f.data_ptr(), norm_w.data_ptr(),
+    work = torch.empty((T, H * dv + H), dtype=torch.float32, device=proj.device)     # read-outs, then denominators
+    _call(entry, proj.data_ptr(), proj.shape[1], bias_i.data_ptr(), bias_f.data_ptr(), norm_w.data_ptr(),
           dtype_code(norm_w.dtype), out.data_ptr(), dtype_code(out.dtype), work.data_ptr(), cu_seqlens.data_ptr(),
           slots.data_ptr(), S.data_ptr(), n.data_ptr(), m.data_ptr(), T, int(n_seqs), int(n_slots), H, d, dv, float(cap),
           float(eps), _stream())
@@ -678,6 +688,19 @@ def gelu_mul_rows(z: torch.Tensor, table: torch.Tensor, col0: int, tokens: torch
     _dev(table, "table")
     _call("alice_gelu_mul_rows", z.data_ptr(), dtype_code(z.dtype), table.data_ptr(), dtype_code(table.dtype), table.shape[1],
           int(col0), tokens.data_ptr(), out.data_ptr(), dtype_code(out.dtype), T, n, table.shape[0], int(full_precision), _stream())
+
+
+def head_gate(out: torch.Tensor, out_layout: int, gate: torch.Tensor, T: int, num_heads: int, head_dim: int) -> None:
+    """out[t, h, :] *= sigmoid(gate[t, h]) in place; out: bfloat16 [T, heads * d] row-major, or its flat fragment
+    order; gate: bfloat16 [T, >= heads] with unit column stride (a column slice of a wider tensor)."""
+    if out_layout == LAYOUT_FRAG16:
+        _dev(out, "out", torch.bfloat16, (frag_rows(T) * num_heads * head_dim,))
+    else:
+        _dev(out, "out", torch.bfloat16, (T, num_heads * head_dim))
+    if (not gate.is_cuda or gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.shape[0] != T
+            or gate.shape[1] < num_heads or gate.stride(1) != 1 or gate.stride(0) < num_heads):
+        raise HipLibraryError(f"gate must be [{T}, >= {num_heads}] bfloat16 with unit column stride")
+    _call("alice_head_gate", out.data_ptr(), int(out_layout), gate.data_ptr(), gate.stride(0), T, num_heads, head_dim, _stream())
 
 
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

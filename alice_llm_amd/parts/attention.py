@@ -70,7 +70,7 @@ class Attention(Part):
         # that a run that reads another run's cache finds the layout it expects.
         self.kv_layout = (ops.KV_FRAGMENT if precision.name == "bfloat16" and precision.act == torch.bfloat16
                           and ops.library_ready() and ops.attention_mfma_supported(head_dim)
-                          and score_bias_slopes is None and self.dv == head_dim and not self.n_gate else ops.KV_ROW)
+                          and score_bias_slopes is None and self.dv == head_dim else ops.KV_ROW)
         self._parts: Dict[str, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -141,7 +141,7 @@ class Attention(Part):
         # Single tokens of at most 16 sequences whose keys are split over blocks: the output projection combines the
         # splits itself (one kernel fewer a layer).
         if (ctx.is_decode and self.kv_layout == ops.KV_FRAGMENT and self.o.layout == ops.LAYOUT_FRAG16
-                and self.nH // self.nKV <= 16 and getattr(ctx, "fragment_activations", False)):
+                and not self.n_gate and self.nH // self.nKV <= 16 and getattr(ctx, "fragment_activations", False)):
             splits = ops.decode_attention_splits(T, self.nKV, ctx.max_context, self.window)
             slices = ops.linear_parts_slices(T, self.o.n, self.nH, self.d, splits) if splits > 1 else 0
             if slices > 0:

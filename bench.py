@@ -11,6 +11,10 @@ device-to-device copy and a large bfloat16 matrix product of the vendor library)
 of the other configurations: the 2B shape at contexts from 8,000, 16 unequal prompts at the 9B shape, and 8 prompts
 of 6,000 tokens, past the window, at the 27B shape.
 
+    python bench.py --novotar w2048,w4096
+        instead of the above: prefill and decode throughput of the Novotar design at layer sizes of real models
+        (random weights, a few layers), beside Gemma 2 at equal sizes; prints a line of its own
+
 Other runs of the same program:
     python bench.py --preset 9b --batch 16 --prompt-lens uniform:64:2048 --steps 256 --points "" --shapes ""
         16 prompts of unequal, seeded lengths in ragged steps, then 256 decode steps
@@ -104,14 +108,17 @@ def measured_peaks():
 class Run:
     """One model shape with random weights and the measurements on it."""
 
-    def __init__(self, preset, layers, dtype, ids_through_host=False):
+    def __init__(self, preset, layers, dtype, ids_through_host=False, raw=None):
         import torch
         import alice_llm_amd as alice
         self.torch, self.alice = torch, alice
-        raw = alice.preset(preset)
-        self.full_layers = raw["num_hidden_layers"]
-        if layers:
-            raw["num_hidden_layers"] = layers
+        if raw is None:
+            raw = alice.preset(preset)
+            self.full_layers = raw["num_hidden_layers"]
+            if layers:
+                raw["num_hidden_layers"] = layers
+        else:
+            self.full_layers = None
         self.cfg = alice.config_from_dict(raw)
         self.dtype = dtype
         self.elem = 2 if dtype == "bfloat16" else 4
@@ -126,7 +133,7 @@ class Run:
         self.gpu_ms = None
 
     def prompts(self, lens):
-        return [self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen).tolist() for n in lens]
+        return [self.torch.randint(0, self.model.lm.plan.vocab_size, (n,), generator=self.gen).tolist() for n in lens]
 
     def decode(self, lens, steps, warmup, context=0):
         """Prefill prompts of these lengths (in the generation loop's ragged steps), then time `steps` decode steps
@@ -136,8 +143,8 @@ class Run:
         from alice_llm_amd.hip import ops
         batch = len(lens)
         room = [max(n + warmup + steps, context) for n in lens]
-        if max(n + warmup + steps for n in lens) > cfg.max_position_embeddings:
-            raise SystemExit(f"prompt + warmup + steps reach beyond the model's {cfg.max_position_embeddings} positions")
+        if max(n + warmup + steps for n in lens) > self.model.lm.plan.max_positions:
+            raise SystemExit(f"prompt + warmup + steps reach beyond the model's {self.model.lm.plan.max_positions} positions")
         eng = self.model.engine(seq_lens=room, max_seqs=batch)
         slots = eng.open(batch)
         ps = self.prompts(lens)
@@ -232,9 +239,102 @@ class Run:
         torch.cuda.empty_cache()
         return out
 
+    def prefill_batch(self, lens, repeats=3):
+        """Several prompts as one ragged step; the median of `repeats` timings by HIP events, in ms."""
+        torch = self.torch
+        eng = self.model.engine(seq_lens=list(lens), max_seqs=len(lens))
+        ps = self.prompts(lens)
+        gpu = []
+        for it in range(repeats + 1):
+            s = eng.open(len(lens))
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            eng.step(s, ps, "last")
+            b.record()
+            torch.cuda.synchronize()
+            if it:
+                gpu.append(a.elapsed_time(b))
+            eng.close(s)
+        del eng
+        torch.cuda.empty_cache()
+        return sorted(gpu)[len(gpu) // 2]
+
+    def step_bytes(self, contexts):
+        """Bytes a decode step moves whatever the architecture: every weight once, each run's keys and values within
+        its window, and each run's fixed-size state read and written."""
+        total = self.weight_bytes
+        for need in self.model.lm.cache_needs():
+            if need is None:
+                continue
+            if need.kv is not None:
+                for c in contexts:
+                    keys = c if need.kv.window is None else min(c, need.kv.window)
+                    total += keys * need.kv.num_kv_heads * (need.kv.head_dim + need.kv.v_dim) * self.elem
+            for st in need.state:
+                n = 1
+                for x in st.shape:
+                    n *= x
+                total += 2 * n * 4 * len(contexts)
+        return total
+
     def close(self):
         del self.model
         self.torch.cuda.empty_cache()
+
+
+# ---------------------------------------------------------------------------------- Novotar beside Gemma 2
+NOVOTAR_SIZES = {
+    # width, feed-forward, attention heads / kv heads / head size, matrix-memory heads / key size / value size
+    "w2048": dict(width=2048, ff=8192, heads=16, kv=4, dim=128, mheads=8, mdim=128, mvdim=256),
+    "w4096": dict(width=4096, ff=14336, heads=32, kv=8, dim=128, mheads=16, mdim=128, mvdim=256),
+}
+
+
+def novotar_pair_configs(size, vocab=32768, window=1024):
+    """A Novotar configuration of four layers, the middle two run twice (six layer runs), and a Gemma 2 configuration
+    of six layers with the same width, feed-forward, heads, head size, window and vocabulary."""
+    z = NOVOTAR_SIZES[size]
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"], "vdim": z["dim"],
+                                "scale": z["dim"] ** -0.5, "mask": {"size": window}},
+                       "right": {"heads": z["mheads"], "dim": z["mdim"], "vdim": z["mvdim"], "gate_cap": 15.0}},
+             "mlp": {"kind": "dense", "ff": z["ff"], "limit": 7.0}}
+    nov = {"architecture": "Novotar", "vocab": vocab, "width": z["width"], "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+           "layers": [layer] * 4, "loop": {"start": 1, "stop": 3, "times": 2}, "token_side": {"dim": 64}}
+    gem = {"architectures": ["Gemma2ForCausalLM"], "model_type": "gemma2", "vocab_size": vocab, "hidden_size": z["width"],
+           "num_hidden_layers": 6, "num_attention_heads": z["heads"], "num_key_value_heads": z["kv"], "head_dim": z["dim"],
+           "intermediate_size": z["ff"], "max_position_embeddings": 65536, "sliding_window": window,
+           "layer_types": ["sliding_attention"] * 6, "query_pre_attn_scalar": z["dim"],
+           "attn_logit_softcapping": None, "final_logit_softcapping": None, "tie_word_embeddings": False}
+    return nov, gem
+
+
+def novotar_bench(sizes, dtype, steps, warmup):
+    out = {}
+    for size in sizes:
+        if size not in NOVOTAR_SIZES:
+            raise SystemExit(f"--novotar: unknown size '{size}'; known: {sorted(NOVOTAR_SIZES)}")
+        res = {}
+        for name, raw in zip(("novotar", "gemma2"), novotar_pair_configs(size)):
+            run = Run(None, None, dtype, raw=raw)
+            r = {"weights_gb": round(run.weight_bytes / 1e9, 3), "layer_runs": len(run.model.lm.plan.schedule)}
+            for T in (2048, 8192):
+                ms = run.prefill_batch([T])
+                r[f"prefill_{T}"] = {"ms": round(ms, 3), "tok_s": round(T / ms * 1e3, 1)}
+            ms = run.prefill_batch([2048] * 8)
+            r["prefill_8x2048"] = {"ms": round(ms, 3), "tok_s": round(8 * 2048 / ms * 1e3, 1)}
+            for b in (1, 8, 64):
+                dt, c0, c1 = run.decode([2048] * b, steps, warmup)
+                gbs = run.step_bytes([(x + y) // 2 for x, y in zip(c0, c1)]) / (dt / steps) / 1e9
+                r[f"decode_b{b}"] = {"ms_per_step": round(dt / steps * 1e3, 4), "tok_s": round(b * steps / dt, 1),
+                                     "gpu_ms_per_step": round(run.gpu_ms, 4) if run.gpu_ms else None,
+                                     "roofline_gbs": round(gbs, 1), "roofline_frac": round(gbs / PEAK_HBM_GBS, 4)}
+            print(f"[bench] {size} {name}: {r}", file=sys.stderr, flush=True)
+            res[name] = r
+            run.close()
+        out[size] = res
+    return out
 
 
 SHAPES = {
@@ -287,6 +387,8 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", default="2048,8192,512,128", help="prompt lengths whose prefill is timed (the first is the headline's)")
     ap.add_argument("--shapes", default=",".join(SHAPES),
                     help="shorter runs of other configurations, reported under 'shapes' ('' for none)")
+    ap.add_argument("--novotar", default="", help="sizes (w2048,w4096): measure the Novotar design beside Gemma 2 at equal "
+                    "sizes instead of the default workload, and print a line of its own")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own copy and matrix-product rates")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -295,6 +397,13 @@ def main() -> int:
 
     import torch
     torch.cuda.set_device(0)
+    if args.novotar:
+        steps = min(args.steps, 64)
+        res = novotar_bench([x for x in args.novotar.split(",") if x], args.dtype, steps, min(args.warmup, 5))
+        print(json.dumps({"metric": "Novotar beside Gemma 2 at equal layer sizes: prefill and decode, random weights",
+                          "unit": "tokens/s", "n_gpus": 1, "steps": steps, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                          "data": "synthetic (uniform random token ids, random weights)", "sizes": res}), flush=True)
+        return 0
     run = Run(args.preset, args.layers, args.dtype, args.ids_through_host)
     cfg, short = run.cfg, run.short
 
