@@ -150,7 +150,16 @@ __global__ void gelu_mul_rows_kernel(const TZ* __restrict__ z, const TW* __restr
 // read-outs go to a 32-bit workspace and mlstm_finish_kernel norms, weights and gates them.
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ int lds_pad20(int d) { return d + ((84 - d % 64) % 64); }   // stride = 20 mod 64 banks
+// Row strides in LDS, for 32 banks of four bytes read by half a wave at a time.  Q, K and P rows are read as
+// 16 rows x 2 neighbours (operand A, and K as operand B of Q K^T), and K also as 2 rows x 16 neighbours (K'^T V):
+// a stride of 18 mod 32 serves the first without conflicts and the second with two banks shared.  V and S rows
+// are read as 2 rows x 16 neighbours only: 16 mod 32.
+__host__ __device__ __forceinline__ int lds_stride18(int d) { return d + ((18 - d % 32 + 32) % 32); }
+
+// A barrier between phases that exchange data through LDS only: it waits for the wave's LDS accesses, not for its
+// loads and stores of global memory (the rows fetched ahead, the read-outs on their way out), which __syncthreads()
+// would also wait for at every phase.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 constexpr int CTHREADS = 512;     // eight waves a block: two a SIMD, so that one's LDS reads hide behind the other's products
 constexpr int CWAVES = CTHREADS / 64;
@@ -162,10 +171,10 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
     float* __restrict__ S_all, float* __restrict__ n_all, float* __restrict__ m_all,
     int H, int d, int dv, float cap) {
   constexpr int VSS = VS == 32 ? 48 : 80;      // row stride of V and S tiles: 16 mod 64 banks
-  constexpr int PSS = C + 4;
+  constexpr int PSS = C + 2;
   constexpr int CT = C / 16, VT = VS / 16;
   extern __shared__ float lds[];
-  const int QS = lds_pad20(d);
+  const int QS = lds_stride18(d);
   float* Qs = lds;                       // [C][QS]
   float* Ks = Qs + C * QS;               // [C][QS]
   float* Vs = Ks + C * QS;               // [C][VSS]
@@ -240,15 +249,19 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
 
   for (int c0 = t0; c0 < t1; c0 += C) {
     const int len = min(C, t1 - c0);
-    __syncthreads();                                     // the chunk before is done with every buffer
+    lds_barrier();                                     // the chunk before is done with every buffer
     // ---- phase 1: the fetched rows into LDS, the gates' running sums and maxima
 #pragma unroll
     for (int u = 0; u < NQ; ++u) {
       const int i = tid + u * CTHREADS;
       if (i < q4) {
         const int j = i / (d / 4), k = (i % (d / 4)) * 4;
-        *reinterpret_cast<float4*>(Qs + j * QS + k) = float4{rq[u].x * qscale, rq[u].y * qscale, rq[u].z * qscale, rq[u].w * qscale};
-        *reinterpret_cast<float4*>(Ks + j * QS + k) = rk[u];
+        float2* qd = reinterpret_cast<float2*>(Qs + j * QS + k);      // rows start at multiples of 8 bytes
+        float2* kd = reinterpret_cast<float2*>(Ks + j * QS + k);
+        qd[0] = float2{rq[u].x * qscale, rq[u].y * qscale};
+        qd[1] = float2{rq[u].z * qscale, rq[u].w * qscale};
+        kd[0] = float2{rk[u].x, rk[u].y};
+        kd[1] = float2{rk[u].z, rk[u].w};
       }
     }
 #pragma unroll
@@ -269,7 +282,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
     }
     const bool more = c0 + C < t1;
     if (more) fetch(c0 + C);
-    __syncthreads();
+    lds_barrier();
     const float M_last = gM[len - 1], m_last = gm[len - 1];
     // ---- phase 2: P = (Q K^T) . D on and below the diagonal
     for (int tile = wave; tile < CT * (CT + 1) / 2; tile += CWAVES) {
@@ -291,7 +304,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
       }
     }
     if (tid < C) gw[tid] = tid < len ? expf(ga[tid] - M_last) : 0.f;
-    __syncthreads();
+    lds_barrier();
     // ---- phase 3: read-outs coef . Q S_0 + P V, unnormalised; the blocks of a head's first columns also take
     // n . q the same way (n as one more column: Q n_0 and the row sums of P) and leave the denominators
     const int n_tiles3 = CT * VT + (blockIdx.z == 0 ? CT : 0);
@@ -332,7 +345,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
         }
       }
     }
-    __syncthreads();                                     // every read of S_0 and n_0 is over
+    lds_barrier();                                     // every read of S_0 and n_0 is over
     // ---- phase 4: the state at the chunk's end (n again as one more column)
     const float cS = expf(m0 - M_last);
     const int n_tiles4 = (d / 16) * VT + (blockIdx.z == 0 ? d / 16 : 0);
@@ -481,8 +494,8 @@ __global__ void mlstm_finish_kernel(const float* __restrict__ work, const float*
 }
 
 size_t chunk_lds_bytes(int C, int VS, int d) {
-  const int QS = d + ((84 - d % 64) % 64), VSS = VS == 32 ? 48 : 80;
-  return (size_t)(2 * C * QS + C * VSS + C * (C + 4) + d * VSS + d + 5 * C) * sizeof(float);
+  const int QS = lds_stride18(d), VSS = VS == 32 ? 48 : 80;
+  return (size_t)(2 * C * QS + C * VSS + C * (C + 2) + d * VSS + d + 5 * C) * sizeof(float);
 }
 
 // The chunk length and the columns a block owns for these sizes (0, 0: the chunk kernel does not cover them).

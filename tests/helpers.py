@@ -168,7 +168,38 @@ def _nv_c():
             "loop": {"start": 0, "stop": 2, "times": 3}, "token_side": {"dim": 16}}
 
 
-NOVOTAR = {"nv-a": _nv_a, "nv-b": _nv_b, "nv-c": _nv_c}
+# D: sizes that fit no tile anywhere (width 72, heads of 20 / 28 / 12, a side input of 5), one kv head for three
+#    query heads, a loop over the first layer alone, a layer without a window.
+def _nv_d():
+    le = {"heads": 3, "kv_heads": 1, "dim": 20, "vdim": 28, "scale": 0.25, "mask": {"size": 33}}
+    ri = {"heads": 2, "dim": 12, "vdim": 20, "gate_cap": 6.0}
+    mlp = {"kind": "dense", "ff": 100, "limit": 2.5}
+    free = {k: v for k, v in le.items() if k != "mask"}
+    return {"architecture": "Novotar", "vocab": 61, "width": 72, "embedding": {"scale": 3.0}, "norm": {"eps": 1e-6},
+            "layers": [_nv_layer(le, ri, mlp), _nv_layer(free, ri, mlp)],
+            "loop": {"start": 0, "stop": 1, "times": 2}, "token_side": {"dim": 5}}
+
+
+NOVOTAR = {"nv-a": _nv_a, "nv-b": _nv_b, "nv-c": _nv_c, "nv-d": _nv_d}
+
+
+def novotar_folder(name: str, seed: int = 0) -> str:
+    """A model folder (config.json, model.safetensors in bfloat16) of a Novotar test configuration."""
+    global _TMP
+    key = ("novotar", name, seed)
+    if key not in _FOLDERS:
+        from safetensors.torch import save_file
+        if _TMP is None:
+            _TMP = tempfile.TemporaryDirectory(prefix="alice_tests_")
+        folder = os.path.join(_TMP.name, f"{name}-{seed}")
+        os.makedirs(folder, exist_ok=True)
+        raw = NOVOTAR[name]()
+        _, tensors = novotar_tensors(raw, seed)
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(raw, f)
+        save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
+        _FOLDERS[key] = folder
+    return _FOLDERS[key]
 
 
 def novotar_tensors(raw: dict, seed: int):

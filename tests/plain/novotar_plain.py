@@ -131,9 +131,10 @@ def matrix_memory(h, w, *, heads, dim, vdim, cap, eps, state=None, return_state=
 
 def parallel_mixer(h, w_left, w_right, left, right, eps):
     """Half the sum of the two sides, each RMS-normed over the width with its own plain weight."""
-    a = gated_attention(h, w_left, heads=left["heads"], kv_heads=left["kv_heads"], dim=left["dim"],
-                        vdim=left["vdim"], scale=left["scale"], window=left["mask"]["size"])
-    b = matrix_memory(h, w_right, heads=right["heads"], dim=right["dim"], vdim=right["vdim"],
+    a = gated_attention(h, w_left, heads=left["heads"], kv_heads=left.get("kv_heads", left["heads"]), dim=left["dim"],
+                        vdim=left.get("vdim", left["dim"]), scale=left["scale"],
+                        window=left["mask"]["size"] if left.get("mask") else h.shape[0])
+    b = matrix_memory(h, w_right, heads=right["heads"], dim=right["dim"], vdim=right.get("vdim", right["dim"]),
                       cap=right["gate_cap"], eps=eps)
     return 0.5 * (rms_norm(a, w_left["out"], eps) + rms_norm(b, w_right["out"], eps))
 

@@ -2,7 +2,10 @@
 model through the engine: whole prompts, a prefix and then single tokens, prompts in pieces down to two tokens,
 unequal batches against each request alone on slots and pages that are used again, long decoding from the first
 token, and greedy generation through the package's own entry point."""
-import math
+import json
+import os
+import subprocess
+import sys
 
 import pytest
 import torch
@@ -12,7 +15,7 @@ from alice_llm_amd.cache import Cache
 from alice_llm_amd.hip import ops
 from alice_llm_amd.parts import FEED_FORWARDS, MIXERS, Precision
 from alice_llm_amd.engine.step import StepContext
-from helpers import NOVOTAR, max_err, novotar_pair, random_tokens
+from helpers import NOVOTAR, max_err, novotar_folder, novotar_pair, random_tokens
 from plain import novotar_plain as P
 
 pytestmark = pytest.mark.gpu
@@ -397,3 +400,53 @@ def test_greedy_generation_through_the_entry_point(name, dtype):
                 assert float(lg.max() - lg[tok]) < 0.15 * float(lg.std()) + 0.05
             seq.append(tok)
     model.release_engine()
+
+
+# ------------------------------------------------------------------ a folder on disk: loader, command line, trace replay
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_replay_of_a_folder(dtype, tmp_path):
+    """bin/trace_run on a model folder: prompts of unequal lengths as one batch, single tokens together, a request
+    that ends early, one that starts later on the slot given back; rows asked for by index."""
+    from plain.novotar_plain import PlainNovotar
+    folder = novotar_folder("nv-d", 5)
+    plain = PlainNovotar.from_folder(folder)
+    a, b, c = (random_tokens(61, n, 60 + n) for n in (70, 9, 40))
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:66], "want": [0, 64, 65]}, {"id": "b", "tokens": b[:7], "want": [6]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[66:67], "want": [0]}, {"id": "b", "tokens": b[7:8], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[67:68], "want": []}, {"id": "b", "tokens": b[8:9], "want": [0]}], "end": ["b"]},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[68:69], "want": [0]}], "end": []},
+             {"step": 4, "entries": [{"id": "c", "tokens": c[:38], "want": [37]}], "end": []},
+             {"step": 5, "entries": [{"id": "c", "tokens": c[38:], "want": [0, 1]}], "end": ["c"]},
+             {"step": 6, "entries": [{"id": "a", "tokens": a[69:], "want": [0]}], "end": ["a"]}]
+    out = tmp_path / "out"
+    proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
+                           "--max-tokens", "140"], input="".join(json.dumps(s) + "\n" for s in steps),
+                          capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == [f"done {i}" for i in range(7)]
+    ra, rb, rc = plain.forward(a), plain.forward(b), plain.forward(c)
+    want = {0: torch.stack([ra[0], ra[64], ra[65], rb[6]]), 1: torch.stack([ra[66], rb[7]]), 2: rb[8][None], 3: ra[68][None],
+            4: rc[37][None], 5: torch.stack([rc[38], rc[39]]), 6: ra[69][None]}
+    got_all, want_all = [], []
+    for i, w in want.items():
+        got = torch.frombuffer(bytearray((out / f"{i}.f32").read_bytes()), dtype=torch.float32).view(-1, 61)
+        assert got.shape == w.shape, i
+        got_all.append(got)
+        want_all.append(w)
+    assert_close(torch.cat(got_all), torch.cat(want_all), dtype)
+
+
+def test_command_line_generates_from_a_folder():
+    from plain.novotar_plain import PlainNovotar
+    folder = novotar_folder("nv-a", 6)
+    plain = PlainNovotar.from_folder(folder)
+    proc = subprocess.run([sys.executable, "-m", "alice_llm_amd.generate", "--model", folder, "--dtype", "float32",
+                           "--prompt-ids", "5,9,11,60", "--prompt-ids", "3", "--max-tokens", "5"],
+                          capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    for prompt in ([5, 9, 11, 60], [3]):
+        ids = plain.greedy(prompt, 5)
+        assert ",".join(str(i) for i in ids) in proc.stdout, (ids, proc.stdout[-500:])
