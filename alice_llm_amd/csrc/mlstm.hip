@@ -20,6 +20,7 @@
 
 namespace {
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 constexpr int THREADS = 256;
 constexpr int MAXC = 4;          // value columns a thread owns at most (dv <= MAXC * 256)
 
@@ -148,7 +149,6 @@ __global__ void gelu_mul_rows_kernel(const TZ* __restrict__ z, const TW* __restr
 // A block owns VS of a head's value columns (S's columns are independent of each other) for all chunks of
 // one sequence; blocks of one head recompute its gates and Q K^T.  The head norm needs every column, so the
 // read-outs go to a 32-bit workspace and mlstm_finish_kernel norms, weights and gates them.
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // Row strides in LDS, for 32 banks of four bytes read by half a wave at a time.  Q, K and P rows are read as
 // 16 rows x 2 neighbours (operand A, and K as operand B of Q K^T), and K also as 2 rows x 16 neighbours (K'^T V):
@@ -161,6 +161,23 @@ __host__ __device__ __forceinline__ int lds_stride18(int d) { return d + ((18 - 
 // would also wait for at every phase.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// acc += sum over k < n (a multiple of 16) of A(k) B(k), four k at a time, as four chains of products that do not
+// wait for each other (a product that adds to the one before it waits for its result, about twice the time the
+// matrix unit is busy with it); the chains are added at the end.
+template <class FA, class FB>
+__device__ __forceinline__ void mfma_chains(f32x4_t& acc, int n, FA a, FB b) {
+  f32x4_t c1 = {0.f, 0.f, 0.f, 0.f}, c2 = c1, c3 = c1;
+#pragma unroll 2
+  for (int kk = 0; kk < n; kk += 16) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a(kk), b(kk), acc, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a(kk + 4), b(kk + 4), c1, 0, 0, 0);
+    c2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a(kk + 8), b(kk + 8), c2, 0, 0, 0);
+    c3 = __builtin_amdgcn_mfma_f32_16x16x4f32(a(kk + 12), b(kk + 12), c3, 0, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] += (c1[i] + c2[i]) + c3[i];
+}
+
 constexpr int CTHREADS = 512;     // eight waves a block: two a SIMD, so that one's LDS reads hide behind the other's products
 constexpr int CWAVES = CTHREADS / 64;
 
@@ -170,7 +187,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
     float* __restrict__ work, float* __restrict__ dens, const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
     float* __restrict__ S_all, float* __restrict__ n_all, float* __restrict__ m_all,
     int H, int d, int dv, float cap) {
-  constexpr int VSS = VS == 32 ? 48 : 80;      // row stride of V and S tiles: 16 mod 64 banks
+  constexpr int VSS = VS == 16 ? 16 : VS + 16; // row stride of V and S tiles: 16 mod 32 banks
   constexpr int PSS = C + 2;
   constexpr int CT = C / 16, VT = VS / 16;
   extern __shared__ float lds[];
@@ -292,8 +309,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
       const float* qa = Qs + (ti * 16 + (lane & 15)) * QS + (lane >> 4);
       const float* kb = Ks + (tj * 16 + (lane & 15)) * QS + (lane >> 4);
-#pragma unroll 8
-      for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], kb[kk], acc, 0, 0, 0);
+      mfma_chains(acc, d, [&](int k) { return qa[k]; }, [&](int k) { return kb[k]; });
       const int r = tj * 16 + (lane & 15);
       const float ar = ga[r];
 #pragma unroll
@@ -317,13 +333,11 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
       const float* pa = Ps + (ti * 16 + (lane & 15)) * PSS + (lane >> 4);
       if (!is_n) {
         const float* sb = Ss + (lane >> 4) * VSS + tn * 16 + (lane & 15);
-#pragma unroll 8
-        for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], sb[kk * VSS], acc, 0, 0, 0);
+        mfma_chains(acc, d, [&](int k) { return qa[k]; }, [&](int k) { return sb[k * VSS]; });
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] *= gcoef[ti * 16 + (lane >> 4) * 4 + i];
         const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
-#pragma unroll 4
-        for (int kk = 0; kk < (ti + 1) * 16; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[kk], vb[kk * VSS], acc, 0, 0, 0);
+        mfma_chains(acc, (ti + 1) * 16, [&](int k) { return pa[k]; }, [&](int k) { return vb[k * VSS]; });
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int j = ti * 16 + (lane >> 4) * 4 + i;
@@ -331,13 +345,11 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
         }
       } else {
         const float* nb = n0 + (lane >> 4);
-#pragma unroll 8
-        for (int kk = 0; kk < d; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk], col0 ? nb[kk] : 0.f, acc, 0, 0, 0);
+        mfma_chains(acc, d, [&](int k) { return qa[k]; }, [&](int k) { return col0 ? nb[k] : 0.f; });
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] *= gcoef[ti * 16 + (lane >> 4) * 4 + i];
         const float one = col0 ? 1.f : 0.f;
-#pragma unroll 4
-        for (int kk = 0; kk < (ti + 1) * 16; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[kk], one, acc, 0, 0, 0);
+        mfma_chains(acc, (ti + 1) * 16, [&](int k) { return pa[k]; }, [&](int) { return one; });
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int j = ti * 16 + (lane >> 4) * 4 + i;
@@ -360,9 +372,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] = cS * sp[i * VSS];
         const float* vb = Vs + (lane >> 4) * VSS + tn * 16 + (lane & 15);
-#pragma unroll 8
-        for (int kk = 0; kk < C; kk += 4)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kk * QS] * gw[kk + (lane >> 4)], vb[kk * VSS], acc, 0, 0, 0);
+        mfma_chains(acc, C, [&](int k) { return ka[k * QS] * gw[k + (lane >> 4)]; }, [&](int k) { return vb[k * VSS]; });
 #pragma unroll
         for (int i = 0; i < 4; ++i) sp[i * VSS] = acc[i];
       } else {
@@ -370,9 +380,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] = col0 ? cS * np[i] : 0.f;
         const float one = col0 ? 1.f : 0.f;
-#pragma unroll 8
-        for (int kk = 0; kk < C; kk += 4)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[kk * QS] * gw[kk + (lane >> 4)], one, acc, 0, 0, 0);
+        mfma_chains(acc, C, [&](int k) { return ka[k * QS] * gw[k + (lane >> 4)]; }, [&](int) { return one; });
         if (col0) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) np[i] = acc[i];
@@ -494,7 +502,7 @@ __global__ void mlstm_finish_kernel(const float* __restrict__ work, const float*
 }
 
 size_t chunk_lds_bytes(int C, int VS, int d) {
-  const int QS = lds_stride18(d), VSS = VS == 32 ? 48 : 80;
+  const int QS = lds_stride18(d), VSS = VS == 16 ? 16 : VS + 16;
   return (size_t)(2 * C * QS + C * VSS + C * (C + 2) + d * VSS + d + 5 * C) * sizeof(float);
 }
 
