@@ -47,6 +47,15 @@ int alice_add_norm(float* resid, const float* branch, int n_partials, long parti
                    const int* rows, int T, int H, float eps_post, float eps_pre, float off_post,
                    float off_pre, int full_precision, int out_layout, hipStream_t stream);
 
+// resid += sum over n branches of norm_j(sum of the branch's partial results), norm_j(b) = b / sqrt(mean(b^2) +
+// eps_j) * (offsets_j + weights_j) where weights_j is given and b itself where it is null; out (optional): the new
+// rows in out_dtype.  The arrays are read on the host.
+#define ALICE_MAX_BRANCHES 4
+int alice_add_branches(float* resid, int n, const float* const* branches, const int* n_partials,
+                       const long* partial_strides, const void* const* weights, int w_dtype, const float* eps,
+                       const float* offsets, void* out, int out_dtype, int T, int H, int full_precision,
+                       hipStream_t stream);
+
 int alice_softcap(float* x, long n, float cap, int full_precision, hipStream_t stream);
 
 // y[M, N] = x[M, K] . W^T with an optional epilogue.  `variant` forces a kernel (tests); AUTO picks.
@@ -106,10 +115,12 @@ long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 // = (maximum as a base-2 exponent, sum, two unused, unnormalised output: the output starts at a multiple of 16
 // bytes), for alice_linear_parts to combine.
 #define ALICE_ATTN_PARTS_HEAD 4
+// gate (optional, with splits > 1 and an output): bfloat16 rows of gate_stride elements whose first nH hold one
+// number a head; head h's output is multiplied by sigmoid(gate[b * gate_stride + h]) where the splits are combined.
 int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
                            const int* context_lens, const int* block_table, int bt_stride, int B, int nH,
                            int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
-                           int out_layout, hipStream_t stream);
+                           int out_layout, const void* gate, int gate_stride, hipStream_t stream);
 
 // The output projection straight from the parts of alice_attention_decode (at most 16 sequences and 16 splits, weights in the
 // fragment layout, [N, nH d]): y[slices][M][N] float32 partial sums, slices = alice_linear_parts_split(...), which

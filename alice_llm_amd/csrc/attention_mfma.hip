@@ -688,7 +688,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 // splits in the order 0, 1, ..., eight loads in flight at a time (a loop of dependent round trips to memory
 // would cost more than the arithmetic).
 __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out, int D, int splits,
-                                          int nH, int out_layout) {
+                                          int nH, int out_layout, const bf16_t* __restrict__ gate, int gate_stride) {
   __shared__ float fs[65];
   const int PS = D + ALICE_ATTN_PARTS_HEAD;
   const float* pr = parts + (size_t)blockIdx.x * splits * PS;
@@ -703,7 +703,9 @@ __global__ void attn_decode_reduce_kernel(const float* __restrict__ parts, bf16_
     if (t == 0) fs[64] = ll;
   }
   __syncthreads();
-  const float inv = 1.f / fs[64];
+  // one gate number a head (optional): the head's output times its sigmoid
+  const float gs = gate ? 1.f / (1.f + __expf(-bf16_to_f32(gate[(size_t)(blockIdx.x / nH) * gate_stride + blockIdx.x % nH]))) : 1.f;
+  const float inv = gs / fs[64];
   for (int e = t; e < D; e += blockDim.x) {
     float acc = 0.f;
     for (int s0 = 0; s0 < splits; s0 += 8) {
@@ -859,12 +861,13 @@ extern "C" long alice_attention_decode_workspace(int B, int nH, int d, int split
 extern "C" int alice_attention_decode(const void* q, const void* k_pool, const void* v_pool, void* out, float* parts,
                                       const int* context_lens, const int* block_table, int bt_stride, int B, int nH,
                                       int nKV, int d, int page_size, float scale, float softcap, int window, int splits,
-                                      int out_layout, hipStream_t stream) {
+                                      int out_layout, const void* gate, int gate_stride, hipStream_t stream) {
   ALICE_CHECK(alice_attention_mfma_supported(d), "attention (matrix cores): head_dim %d is not covered (64, 128 or 256)", d);
   ALICE_CHECK(nKV >= 1 && nH % nKV == 0 && nH / nKV <= 16, "attention (decode): %d query heads per kv head are more than the 16 this kernel takes", nKV ? nH / nKV : 0);
   ALICE_CHECK(page_size == 64, "attention (matrix cores): pages must hold 64 positions, found %d", page_size);
   ALICE_CHECK(B >= 0 && nKV <= 65535 && splits >= 1 && splits <= 64, "attention: bad batch B=%d or splits=%d", B, splits);
   ALICE_CHECK(splits == 1 || parts != nullptr, "attention: split keys need the workspace");
+  ALICE_CHECK(gate == nullptr || (splits > 1 && out != nullptr && gate_stride >= nH), "attention (decode): the gate is applied where the key splits are combined (splits > 1, with an output)");
   ALICE_CHECK(out != nullptr || splits > 1, "attention: without an output the keys must be split (the parts are the result)");
   ALICE_CHECK(softcap >= 0.f && window >= 0 && bt_stride > 0, "attention: bad softcap, window or block table");
   ALICE_CHECK(out_layout == 0 || out_layout == 1, "attention: unknown output layout %d", out_layout);
@@ -897,7 +900,8 @@ extern "C" int alice_attention_decode(const void* q, const void* k_pool, const v
 #undef GO1
   ALICE_LAUNCH_CHECK();
   if (splits > 1 && out != nullptr) {
-    attn_decode_reduce_kernel<<<B * nH, d <= 64 ? 64 : 128, 0, stream>>>(parts, (bf16_t*)out, d, splits, nH, out_layout);
+    attn_decode_reduce_kernel<<<B * nH, d <= 64 ? 64 : 128, 0, stream>>>(parts, (bf16_t*)out, d, splits, nH, out_layout,
+                                                                         (const bf16_t*)gate, gate_stride);
     ALICE_LAUNCH_CHECK();
   }
   return 0;

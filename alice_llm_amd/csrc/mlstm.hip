@@ -479,6 +479,74 @@ __global__ __launch_bounds__(THREADS) void mlstm_cols_kernel(
   }
 }
 
+
+// Single tokens with value heads of up to 256 and keys of up to 128: a block per (sequence, head), a thread per
+// value column with the column's d elements of S in registers.  The head's read-out is whole inside the block, so
+// the head norm, its weight and the output gate follow at once: one kernel a step, the state read and written once.
+template <int DMAX, typename TO>
+__global__ __launch_bounds__(THREADS) void mlstm_head_kernel(
+    const float* __restrict__ proj, int row_w, const float* __restrict__ bias_i, const float* __restrict__ bias_f,
+    const void* __restrict__ norm_w, int norm_dtype, TO* __restrict__ out, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, float* __restrict__ S_all, float* __restrict__ n_all, float* __restrict__ m_all,
+    int H, int d, int dv, float cap, float eps) {
+  extern __shared__ float lds[];
+  float* qs = lds;                 // d
+  float* ks = qs + d;              // d
+  float* ns = ks + d;              // d
+  __shared__ float red[17];
+  const int s = blockIdx.x, h = blockIdx.y, c = threadIdx.x;
+  const bool col = c < dv;
+  const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
+  if (t1 <= t0) return;
+  const int slot = slots[s];
+  float* S = S_all + ((size_t)slot * H + h) * d * dv;
+  float* ng = n_all + ((size_t)slot * H + h) * d;
+  float m = m_all[(size_t)slot * H + h];
+  float st[DMAX];
+#pragma unroll
+  for (int r = 0; r < DMAX; ++r) st[r] = (col && r < d) ? S[(size_t)r * dv + c] : 0.f;
+  for (int r = c; r < d; r += blockDim.x) ns[r] = ng[r];
+  const float qscale = rsqrtf((float)d);
+  const int oq = h * d, ok = H * d + h * d, ov = 2 * H * d + h * dv, og = 2 * H * d + H * dv + h * dv;
+  const int oa = 2 * H * d + 2 * H * dv + h, ob = oa + H;
+  const float bi = bias_i[h], bf = bias_f[h];
+  const float w = !col ? 0.f : norm_dtype == DT_F32 ? ((const float*)norm_w)[h * dv + c] : bf16_to_f32(((const bf16_t*)norm_w)[h * dv + c]);
+  for (int t = t0; t < t1; ++t) {
+    const float* row = proj + (size_t)t * row_w;
+    __syncthreads();
+    for (int r = c; r < d; r += blockDim.x) { qs[r] = row[oq + r] * qscale; ks[r] = row[ok + r]; }
+    const float v = col ? row[ov + c] : 0.f, g = col ? row[og + c] : 0.f;
+    const GateNumbers gn = gate_numbers(row[oa] + bi, row[ob] + bf, cap, m);
+    __syncthreads();
+    float nq = 0.f;
+    for (int r = c; r < d; r += blockDim.x) {
+      const float x = fmaf(gn.keep, ns[r], gn.put * ks[r]);
+      ns[r] = x;
+      nq = fmaf(x, qs[r], nq);
+    }
+    nq = block_sum(nq, red);
+    const float pv = gn.put * v;
+    float acc = 0.f;
+#pragma unroll
+    for (int r = 0; r < DMAX; ++r) {
+      if (r < d) {
+        st[r] = fmaf(gn.keep, st[r], ks[r] * pv);
+        acc = fmaf(st[r], qs[r], acc);
+      }
+    }
+    const float o = col ? acc / (fmaxf(fabsf(nq), expf(-gn.m_new)) + 1e-6f) : 0.f;
+    const float sq = block_sum(o * o, red);
+    if (col) store_f32(out, (size_t)t * H * dv + h * dv + c, o / sqrtf(sq / (float)dv + eps) * w / (1.f + expf(-g)));
+    m = gn.m_new;
+  }
+#pragma unroll
+  for (int r = 0; r < DMAX; ++r)
+    if (col && r < d) S[(size_t)r * dv + c] = st[r];
+  __syncthreads();
+  for (int r = c; r < d; r += blockDim.x) ng[r] = ns[r];
+  if (c == 0) m_all[(size_t)slot * H + h] = m;
+}
+
 // With o = work[t, h, :] (divided by dens[t, h] where the read-outs were left unnormalised):
 // out[t, h, :] = o / rms(o) * w[h, :] * sigmoid(g[t, h, :]); a block per (token, head).
 template <typename TO>
@@ -573,8 +641,9 @@ extern "C" int alice_gelu_mul_rows(const void* z, int z_dtype, const void* table
   return 0;
 }
 
-// alice_mlstm_step's result for key sizes up to 256 with the state read and written once a step, in blocks of 64
-// value columns; work: float32 [T, H * dv].
+// alice_mlstm_step's result for key sizes up to 256 with the state read and written once a step: a block a head
+// where the head fits one (keys up to 128, values up to 256), else blocks of 64 value columns and a finishing
+// kernel; work: float32 [T, H * dv].
 extern "C" int alice_mlstm_cols(const float* proj, int row_w, const float* bias_i, const float* bias_f,
                                 const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
                                 const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
@@ -587,6 +656,19 @@ extern "C" int alice_mlstm_cols(const float* proj, int row_w, const float* bias_
   ALICE_CHECK(proj && bias_i && bias_f && norm_w && out && work && cu_seqlens && slots && S && n && m && n_slots >= 1,
               "mlstm: a pointer is missing");
   if (n_seqs == 0 || T == 0) return 0;
+  // The whole head in one block (no workspace, no second kernel) where such blocks fill the chip; with fewer, a
+  // CU's own share of the memory rate bounds a block that moves a whole head's state (batch 8 of 8 heads: 24 us
+  // against 11 + 9 for the two kernels below).
+  if (d <= 128 && dv <= THREADS && (long)n_seqs * H >= 256) {
+    const int threads = (dv + 63) / 64 * 64;
+    const size_t lds1 = (size_t)3 * d * sizeof(float);
+#define GO1(D, TT) mlstm_head_kernel<D, TT><<<dim3(n_seqs, H), threads, lds1, stream>>>(proj, row_w, bias_i, bias_f, norm_w, norm_dtype, (TT*)out, cu_seqlens, slots, S, n, m, H, d, dv, cap, eps)
+    if (out_dtype == DT_F32) { if (d <= 32) GO1(32, float); else if (d <= 64) GO1(64, float); else GO1(128, float); }
+    else { if (d <= 32) GO1(32, bf16_t); else if (d <= 64) GO1(64, bf16_t); else GO1(128, bf16_t); }
+#undef GO1
+    ALICE_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid(n_seqs, H, (dv + 63) / 64);
   const size_t lds = (size_t)(3 * d + 256) * sizeof(float);
 #define GO(R) mlstm_cols_kernel<R><<<grid, THREADS, lds, stream>>>(proj, row_w, bias_i, bias_f, work, cu_seqlens, slots, S, n, m, H, d, dv, cap)

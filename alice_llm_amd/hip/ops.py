@@ -39,6 +39,7 @@ def _declare(lib) -> None:
         "alice_embed": [P, P, I, I, P, I, I, I, F, P],
         "alice_add_norm": [P, P, I, L, P, P, I, P, I, P, I, I, F, F, F, F, I, I, P],
         "alice_softcap": [P, L, F, I, P],
+        "alice_add_branches": [P, I, P, P, P, P, I, P, P, P, I, I, I, I, P],
         "alice_linear": [P, I, P, I, I, P, I, I, I, I, I, F, I, I, I, I, I, P],
         "alice_linear_split_hint": [I, I, I, I],
         "alice_to_frag16": [P, P, I, I, P],
@@ -52,7 +53,7 @@ def _declare(lib) -> None:
         "alice_linear_rope_cache": [P, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_attention_mfma_supported": [I],
         "alice_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
-        "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P],
+        "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, P],
         "alice_head_gate": [P, I, P, I, I, I, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
@@ -232,6 +233,38 @@ def add_norm(resid: torch.Tensor, branch: Optional[torch.Tensor], w_post: Option
           _opt(out, "out"), dtype_code(out.dtype if out is not None else torch.float32),
           _opt(rows, "rows"), T, H, float(eps_post), float(eps_pre), float(off_post), float(off_pre),
           int(full_precision), int(out_layout), _stream())
+
+
+MAX_BRANCHES = 4
+ADD_BRANCHES_MAX_WIDTH = 8192      # rows that add_branches holds in registers
+
+
+def add_branches(resid: torch.Tensor, branches, out: Optional[torch.Tensor] = None, *, full_precision: bool) -> None:
+    """resid += sum of norm_j(branch_j) in one kernel.  branches: up to four (tensor, weight, eps, offset) with tensor
+    float32 [T, H] or [S, T, H] partial results; weight None adds the branch as it is, else it is RMS-normed over
+    the row first and multiplied by (offset + weight).  out (optional): the new rows in its own dtype, [T, H]."""
+    T, H = resid.shape
+    _dev(resid, "resid", torch.float32)
+    n = len(branches)
+    if not 1 <= n <= MAX_BRANCHES:
+        raise HipLibraryError(f"add_branches takes 1 to {MAX_BRANCHES} branches, found {n}")
+    c = ctypes
+    ptrs, parts, strides, ws, eps, offs = (c.c_void_p * n)(), (c.c_int * n)(), (c.c_long * n)(), (c.c_void_p * n)(), (c.c_float * n)(), (c.c_float * n)()
+    w_dtype = None
+    for j, (b, w, e, o) in enumerate(branches):
+        p = b.shape[0] if b.dim() == 3 else 1
+        _dev(b, "branch", torch.float32, (p, T, H) if b.dim() == 3 else (T, H))
+        ptrs[j], parts[j], strides[j] = b.data_ptr(), p, T * H
+        if w is not None:
+            _dev(w, "weight", None, (H,))
+            if w_dtype is not None and w.dtype != w_dtype:
+                raise HipLibraryError("the branches' norm weights must have one dtype")
+            w_dtype = w.dtype
+        ws[j], eps[j], offs[j] = (None if w is None else w.data_ptr()), float(e), float(o)
+    if out is not None:
+        _dev(out, "out", None, (T, H))
+    _call("alice_add_branches", resid.data_ptr(), n, ptrs, parts, strides, ws, dtype_code(w_dtype or torch.float32), eps, offs,
+          _opt(out, "out"), dtype_code(out.dtype if out is not None else torch.float32), T, H, int(full_precision), _stream())
 
 
 def frag_rows(rows: int) -> int:
@@ -490,8 +523,10 @@ def attention_prefill(q, k_pool, v_pool, out, cu_seqlens, context_lens, block_ta
 
 def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_heads: int, max_context: int,
                      scale: float, softcap: Optional[float], window: Optional[int], splits: Optional[int] = None,
-                     out_layout: int = LAYOUT_ROW):
-    """out_layout FRAG16: `out` is a flat buffer of ceil16(B) * num_heads * d elements in fragment order.
+                     out_layout: int = LAYOUT_ROW, gate: Optional[torch.Tensor] = None):
+    """gate: bfloat16 [B, >= heads] with unit column stride; applied where the key splits are combined (so only with
+    splits > 1 and an output; returns False in the third place otherwise and the caller gates the output itself).
+    out_layout FRAG16: `out` is a flat buffer of ceil16(B) * num_heads * d elements in fragment order.
     Returns (parts, splits).  With out=None the keys' splits are left uncombined in `parts`
     ([B, heads, splits, 4 + d] float32, flat) for linear_parts(); that needs splits > 1."""
     n_pages, nKV, page_size, d = k_pool.shape
@@ -516,9 +551,18 @@ def attention_decode(q, k_pool, v_pool, out, context_lens, block_table, *, num_h
         raise HipLibraryError("attention_decode: without an output buffer the keys must be split")
     parts = (torch.empty((library().alice_attention_decode_workspace(B, num_heads, d, splits),), dtype=torch.float32,
                          device=q.device) if splits > 1 else None)
+    gate_ptr, gate_stride = None, 0
+    if gate is not None and splits > 1 and out is not None:
+        if (not gate.is_cuda or gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.shape[0] != B
+                or gate.shape[1] < num_heads or gate.stride(1) != 1 or gate.stride(0) < num_heads):
+            raise HipLibraryError(f"gate must be [{B}, >= {num_heads}] bfloat16 with unit column stride")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
     _call("alice_attention_decode", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), None if out is None else out.data_ptr(),
           _opt(parts, "parts"), context_lens.data_ptr(), block_table.data_ptr(), block_table.shape[1], B, num_heads,
-          nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), splits, int(out_layout), _stream())
+          nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0), splits, int(out_layout),
+          gate_ptr, int(gate_stride), _stream())
+    if gate is not None:
+        return parts, splits, gate_ptr is not None
     return parts, splits
 
 
@@ -565,9 +609,11 @@ def attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: 
             raise HipLibraryError("the matrix-core attention kernels take no score bias: lay the cache out row-major")
         nKV = k_pool.shape[1]
         if ctx.is_decode and num_heads // nKV <= 16:
-            attention_decode(q, k_pool, v_pool, out, ctx.context_lens, block_table, num_heads=num_heads,
-                             max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
-                             out_layout=out_layout)
+            res = attention_decode(q, k_pool, v_pool, out, ctx.context_lens, block_table, num_heads=num_heads,
+                                   max_context=ctx.max_context, scale=scale, softcap=softcap, window=window,
+                                   out_layout=out_layout, gate=gate)
+            if gate is not None and res[2]:
+                return                                         # gated where the key splits were combined
         else:
             attention_prefill(q, k_pool, v_pool, out, ctx.cu_seqlens, ctx.context_lens, block_table,
                               num_heads=num_heads, n_seqs=ctx.n_seqs, max_new=ctx.max_new,

@@ -58,7 +58,6 @@ class ParallelBlock:
             branches = [(branches, None)]
         if self.feed_forward is not None:
             branches.append((self.feed_forward.forward(h, ctx), None))
-        for branch, post in branches:
-            stream.push(branch, post)
+        stream.push_many(branches)                              # one kernel adds them all
         for extra in self.extras.values():
             extra.forward(stream, ctx)

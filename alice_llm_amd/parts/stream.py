@@ -23,10 +23,34 @@ class ResidualStream:
         self.precision = precision
         self._branch: Optional[torch.Tensor] = None
         self._post = None
+        self._many = None               # several pending branches [(tensor, weight, eps, offset)], added by one kernel
+
+    def push_many(self, branches) -> None:
+        """Queue `x += sum of post_norm_j(branch_j)` for [(branch, post norm or None)]: one kernel adds them all
+        where every norm can be fused (and there are at most ops.MAX_BRANCHES); otherwise one push each."""
+        fused = []
+        for b, post in branches:
+            f = post.fused() if post is not None and hasattr(post, "fused") else None
+            if post is not None and f is None:
+                fused = None
+                break
+            fused.append((b, f[0], f[1], f[2]) if f is not None else (b, None, 0.0, 0.0))
+        dtypes = {w.dtype for _, w, _, _ in (fused or []) if w is not None}
+        if (fused is None or len(fused) > ops.MAX_BRANCHES or len(fused) < 2 or len(dtypes) > 1
+                or self.x.shape[1] > ops.ADD_BRANCHES_MAX_WIDTH):
+            for b, post in branches:
+                self.push(b, post)
+            return
+        self.flush()
+        self._many = fused
+
+    def _flush_many(self, out=None) -> None:
+        ops.add_branches(self.x, self._many, out, full_precision=self.precision.full)
+        self._many = None
 
     def push(self, branch: torch.Tensor, post_norm=None) -> None:
         """Queue `x += post_norm(branch)`.  branch: float32 [T, H], or [S, T, H] partial sums."""
-        if self._branch is not None:
+        if self._branch is not None or self._many is not None:
             self.flush()
         self._branch = branch
         self._post = post_norm
@@ -36,6 +60,8 @@ class ResidualStream:
         return (b.shape[0], b) if b.dim() == 3 else (1, b)
 
     def flush(self) -> None:
+        if self._many is not None:
+            self._flush_many()
         if self._branch is None:
             return
         n, b = self._partials()
@@ -58,6 +84,12 @@ class ResidualStream:
         fragments: the consumer reads fragment order; given where possible (see FragmentActs), else a tensor."""
         out_dtype = out_dtype or self.precision.act
         T, H = self.x.shape
+        if self._many is not None:
+            if norm is None:                                   # the sum and the stream's copy in the activation dtype, one kernel
+                out = torch.empty((T, H), dtype=out_dtype, device=self.x.device)
+                self._flush_many(out)
+                return out
+            self._flush_many()
         pre = norm.fused() if norm is not None and hasattr(norm, "fused") else None
         if fragments and pre is not None and out_dtype == torch.bfloat16 and FragmentActs.possible(self.precision, T, H):
             post = self._post
