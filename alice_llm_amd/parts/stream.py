@@ -16,6 +16,9 @@ from ..hip import ops
 from .base import FragmentActs, Precision
 
 
+ADD_BRANCHES_FROM_ROWS = 256
+
+
 class ResidualStream:
     def __init__(self, x: torch.Tensor, precision: Precision):
         assert x.dtype == torch.float32 and x.dim() == 2
@@ -36,8 +39,11 @@ class ResidualStream:
                 break
             fused.append((b, f[0], f[1], f[2]) if f is not None else (b, None, 0.0, 0.0))
         dtypes = {w.dtype for _, w, _, _ in (fused or []) if w is not None}
+        # Few rows: the single-branch kernel, one launch a branch, is as fast at 8 rows and faster at 64 (a block
+        # of the fused kernel reads every branch's partial results of its row by itself); many rows: one pass
+        # over the stream instead of one a branch.
         if (fused is None or len(fused) > ops.MAX_BRANCHES or len(fused) < 2 or len(dtypes) > 1
-                or self.x.shape[1] > ops.ADD_BRANCHES_MAX_WIDTH):
+                or self.x.shape[1] > ops.ADD_BRANCHES_MAX_WIDTH or self.x.shape[0] < ADD_BRANCHES_FROM_ROWS):
             for b, post in branches:
                 self.push(b, post)
             return
