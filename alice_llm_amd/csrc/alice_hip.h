@@ -4,7 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 7
+#define ALICE_ABI_VERSION 8
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked; epi_param 0: y = gelu_tanh(gate x) * (up x); epi_param = limit > 0:
@@ -142,16 +142,19 @@ int alice_mlstm_step(const float* proj, int row_w, const float* bias_i, const fl
 // alice_mlstm_cols: the same result for single tokens and pieces of a few, key sizes up to 256: a block per
 // (sequence, head, 64 value columns), the state in registers, read and written once a step.
 // The same for steps of many tokens a sequence, a chunk of tokens at a time on the 32-bit matrix instruction;
-// work: T * (H * dv + H) float32 (alice_mlstm_cols: T * H * dv).  alice_mlstm_chunks_supported says whether the head sizes are covered.
+// work: alice_mlstm_chunks_workspace(...) float32 (alice_mlstm_cols: T * H * dv); max_new: the most tokens of one
+// sequence in the step (steps that leave the chip unfilled run their chunks side by side).  alice_mlstm_chunks_supported says whether the head sizes are covered.
 int alice_mlstm_cols(const float* proj, int row_w, const float* bias_i, const float* bias_f,
                      const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
                      const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
                      int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, hipStream_t stream);
 int alice_mlstm_chunks_supported(int n_seqs, int H, int d, int dv);
+long alice_mlstm_chunks_workspace(int T, int n_seqs, int max_new, int H, int d, int dv);
 int alice_mlstm_chunks(const float* proj, int row_w, const float* bias_i, const float* bias_f,
                        const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
                        const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
-                       int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, hipStream_t stream);
+                       int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps, int max_new,
+                       hipStream_t stream);
 
 // out[t, j] = gelu_tanh(z[t, j]) * table[tokens[t], col0 + j], j < n: a gate on columns of a per-token table
 // [V, table_w]; a token outside the table reads zeros.

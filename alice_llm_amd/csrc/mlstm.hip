@@ -181,12 +181,20 @@ __device__ __forceinline__ void mfma_chains(f32x4_t& acc, int n, FA a, FB b) {
 constexpr int CTHREADS = 512;     // eight waves a block: two a SIMD, so that one's LDS reads hide behind the other's products
 constexpr int CWAVES = CTHREADS / 64;
 
-template <int C, int VS>
+// MODE 0: a block walks all chunks of its sequence, from and to the cache's state (grid.x: sequences).
+// For steps whose sequences x heads x slices leave the chip unfilled, the chunks run side by side instead
+// (grid.x: sequences x max_chunks): MODE 1 leaves every chunk's own sums, from an empty state, in the workspace
+// (U = K'^T V with weights exp(a_r - A), A = max_r a_r; u_n alike; A and the chunk's sum of log forget gates);
+// mlstm_chunk_states_kernel walks the chunks' sums and leaves the state and stabiliser before every chunk in
+// their place; MODE 2 takes every chunk's read-outs from the state before it.
+struct ChunkSpace { float* S; float* n; float* sc; float* m0; int max_chunks; };
+
+template <int C, int VS, int MODE>
 __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
     const float* __restrict__ proj, int row_w, const float* __restrict__ bias_i, const float* __restrict__ bias_f,
     float* __restrict__ work, float* __restrict__ dens, const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
     float* __restrict__ S_all, float* __restrict__ n_all, float* __restrict__ m_all,
-    int H, int d, int dv, float cap) {
+    int H, int d, int dv, float cap, ChunkSpace ws) {
   constexpr int VSS = VS == 16 ? 16 : VS + 16; // row stride of V and S tiles: 16 mod 32 banks
   constexpr int PSS = C + 2;
   constexpr int CT = C / 16, VT = VS / 16;
@@ -204,21 +212,25 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
   float* gcoef = gm + C;                 // [C] exp(m_0 - M_j)
   float* gw = gcoef + C;                 // [C] exp(a_r - M_last)
 
-  const int s = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * VS, tid = threadIdx.x;
+  const int s = MODE == 0 ? blockIdx.x : blockIdx.x / ws.max_chunks, chunk = MODE == 0 ? 0 : blockIdx.x % ws.max_chunks;
+  const int h = blockIdx.y, v0 = blockIdx.z * VS, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
-  if (t1 <= t0) return;
+  const int c_begin = t0 + chunk * C, c_end = MODE == 0 ? t1 : min(t1, c_begin + C);
+  if (c_end <= c_begin) return;
   const int slot = slots[s];
-  float* Sg = S_all + ((size_t)slot * H + h) * d * dv;
-  float* ng = n_all + ((size_t)slot * H + h) * d;
-  float m0 = m_all[(size_t)slot * H + h];
+  const size_t cid = (size_t)blockIdx.x * H + h;             // the chunk's place in the workspace (MODE 1, 2)
+  float* Sg = MODE == 0 ? S_all + ((size_t)slot * H + h) * d * dv : ws.S + cid * d * dv;
+  float* ng = MODE == 0 ? n_all + ((size_t)slot * H + h) * d : ws.n + cid * d;
+  float m0 = MODE == 0 ? m_all[(size_t)slot * H + h] : (MODE == 1 ? -INFINITY : ws.m0[cid]);
+  float M_end = 0.f;
   const float qscale = rsqrtf((float)d);
   const int oq = h * d, ok = H * d + h * d, ov = 2 * H * d + h * dv + v0;
   const int oa = 2 * H * d + 2 * H * dv + h, ob = oa + H;
   const float bi = bias_i[h], bf = bias_f[h];
 
-  for (int i = tid; i < d * VS; i += CTHREADS) Ss[(i / VS) * VSS + i % VS] = Sg[(size_t)(i / VS) * dv + v0 + i % VS];
-  for (int r = tid; r < d; r += CTHREADS) n0[r] = ng[r];
+  for (int i = tid; i < d * VS; i += CTHREADS) Ss[(i / VS) * VSS + i % VS] = MODE == 1 ? 0.f : Sg[(size_t)(i / VS) * dv + v0 + i % VS];
+  for (int r = tid; r < d; r += CTHREADS) n0[r] = MODE == 1 ? 0.f : ng[r];
 
   // A chunk's rows are fetched into registers while the chunk before is worked on, and its gates' tanh and
   // logarithm are taken by wave 0 at the end of that chunk: neither waits in a chunk's own time.
@@ -261,10 +273,10 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
       fg_n = logsigmoid_f(cap > 0.f ? cap * tanhf(b / cap) : b);
     }
   };
-  fetch(t0);
-  if (wave == 0) gates_ahead(t0);
+  fetch(c_begin);
+  if (wave == 0) gates_ahead(c_begin);
 
-  for (int c0 = t0; c0 < t1; c0 += C) {
+  for (int c0 = c_begin; c0 < c_end; c0 += C) {
     const int len = min(C, t1 - c0);
     lds_barrier();                                     // the chunk before is done with every buffer
     // ---- phase 1: the fetched rows into LDS, the gates' running sums and maxima
@@ -297,12 +309,12 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
       M = fmaxf(M, m0);
       if (lane < C) { ga[lane] = a; gM[lane] = M; gm[lane] = b + M; gcoef[lane] = expf(m0 - M); }
     }
-    const bool more = c0 + C < t1;
+    const bool more = c0 + C < c_end;
     if (more) fetch(c0 + C);
     lds_barrier();
     const float M_last = gM[len - 1], m_last = gm[len - 1];
     // ---- phase 2: P = (Q K^T) . D on and below the diagonal
-    for (int tile = wave; tile < CT * (CT + 1) / 2; tile += CWAVES) {
+    for (int tile = wave; tile < (MODE == 1 ? 0 : CT * (CT + 1) / 2); tile += CWAVES) {
       int ti = 0, rem = tile;
       while (rem > ti) { rem -= ti + 1; ++ti; }
       const int tj = rem;
@@ -323,7 +335,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
     lds_barrier();
     // ---- phase 3: read-outs coef . Q S_0 + P V, unnormalised; the blocks of a head's first columns also take
     // n . q the same way (n as one more column: Q n_0 and the row sums of P) and leave the denominators
-    const int n_tiles3 = CT * VT + (blockIdx.z == 0 ? CT : 0);
+    const int n_tiles3 = MODE == 1 ? 0 : CT * VT + (blockIdx.z == 0 ? CT : 0);
     for (int tile = wave; tile < n_tiles3; tile += CWAVES) {
       const bool is_n = tile >= CT * VT;
       const int ti = is_n ? tile - CT * VT : tile / VT, tn = is_n ? 0 : tile % VT;
@@ -360,7 +372,7 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
     lds_barrier();                                     // every read of S_0 and n_0 is over
     // ---- phase 4: the state at the chunk's end (n again as one more column)
     const float cS = expf(m0 - M_last);
-    const int n_tiles4 = (d / 16) * VT + (blockIdx.z == 0 ? d / 16 : 0);
+    const int n_tiles4 = MODE == 2 ? 0 : (d / 16) * VT + (blockIdx.z == 0 ? d / 16 : 0);
     for (int tile = wave; tile < n_tiles4; tile += CWAVES) {
       const bool is_n = tile >= (d / 16) * VT;
       const int tk = is_n ? tile - (d / 16) * VT : tile / VT, tn = is_n ? 0 : tile % VT;
@@ -388,14 +400,70 @@ __global__ __launch_bounds__(CTHREADS) void mlstm_chunk_kernel(
       }
     }
     m0 = m_last;
+    M_end = M_last;
     if (more && wave == 0) gates_ahead(c0 + C);
   }
+  if (MODE == 2) return;
   __syncthreads();
   for (int i = tid; i < d * VS; i += CTHREADS) Sg[(size_t)(i / VS) * dv + v0 + i % VS] = Ss[(i / VS) * VSS + i % VS];
   if (blockIdx.z == 0) {
     for (int r = tid; r < d; r += CTHREADS) ng[r] = n0[r];
-    if (tid == 0) m_all[(size_t)slot * H + h] = m0;
+    if (tid == 0) {
+      if (MODE == 0) m_all[(size_t)slot * H + h] = m0;
+      else { ws.sc[cid * 2] = M_end; ws.sc[cid * 2 + 1] = m0 - M_end; }      // A, and the sum of the log forget gates
+    }
   }
+}
+
+// Between MODE 1 and MODE 2: per (sequence, head) the chunks one after the other, element by element.  With the
+// state s and stabiliser m before chunk c, and the chunk's own sums u, A and b: the state before the chunk goes
+// where u was; then M = max(m, A), s <- exp(m - M) s + exp(A - M) u, m <- b + M.  The end state goes to the cache.
+__global__ __launch_bounds__(THREADS) void mlstm_chunk_states_kernel(
+    const int* __restrict__ cu_seqlens, const int* __restrict__ slots, float* __restrict__ S_all,
+    float* __restrict__ n_all, float* __restrict__ m_all, int H, int d, int dv, int C, ChunkSpace ws) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
+  if (t1 <= t0) return;
+  const int n_chunks = (t1 - t0 + C - 1) / C;
+  const int slot = slots[s];
+  const size_t per = (size_t)d * dv;
+  const size_t e = ((size_t)blockIdx.z * THREADS + threadIdx.x) * 4;       // four elements a thread
+  const bool does_n = blockIdx.z == 0 && threadIdx.x < (d + 3) / 4;        // and the first block the vector n too
+  float4 st = {0.f, 0.f, 0.f, 0.f}, nn = st;
+  float* Sg = S_all + ((size_t)slot * H + h) * per;
+  float* ng = n_all + ((size_t)slot * H + h) * d;
+  if (e < per) st = *reinterpret_cast<const float4*>(Sg + e);
+  if (does_n) nn = *reinterpret_cast<const float4*>(ng + threadIdx.x * 4);
+  float m = m_all[(size_t)slot * H + h];
+  for (int c0 = 0; c0 < n_chunks; c0 += 4) {
+    float4 u[4], un[4];
+    float A[4], b[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {                               // the loads of four chunks before the first use
+      const size_t cid = ((size_t)s * ws.max_chunks + min(c0 + k, n_chunks - 1)) * H + h;
+      u[k] = e < per ? *reinterpret_cast<const float4*>(ws.S + cid * per + e) : float4{0.f, 0.f, 0.f, 0.f};
+      un[k] = does_n ? *reinterpret_cast<const float4*>(ws.n + cid * d + threadIdx.x * 4) : float4{0.f, 0.f, 0.f, 0.f};
+      A[k] = ws.sc[cid * 2];
+      b[k] = ws.sc[cid * 2 + 1];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (c0 + k < n_chunks) {
+        const size_t cid = ((size_t)s * ws.max_chunks + c0 + k) * H + h;
+        if (e < per) *reinterpret_cast<float4*>(ws.S + cid * per + e) = st;
+        if (does_n) *reinterpret_cast<float4*>(ws.n + cid * d + threadIdx.x * 4) = nn;
+        if (blockIdx.z == 0 && threadIdx.x == 0) ws.m0[cid] = m;
+        const float M = fmaxf(m, A[k]);
+        const float ka = expf(m - M), kb = expf(A[k] - M);
+        st = float4{ka * st.x + kb * u[k].x, ka * st.y + kb * u[k].y, ka * st.z + kb * u[k].z, ka * st.w + kb * u[k].w};
+        nn = float4{ka * nn.x + kb * un[k].x, ka * nn.y + kb * un[k].y, ka * nn.z + kb * un[k].z, ka * nn.w + kb * un[k].w};
+        m = b[k] + M;
+      }
+    }
+  }
+  if (e < per) *reinterpret_cast<float4*>(Sg + e) = st;
+  if (does_n) *reinterpret_cast<float4*>(ng + threadIdx.x * 4) = nn;
+  if (blockIdx.z == 0 && threadIdx.x == 0) m_all[(size_t)slot * H + h] = m;
 }
 
 
@@ -693,42 +761,77 @@ extern "C" int alice_mlstm_chunks_supported(int n_seqs, int H, int d, int dv) {
 }
 
 // The same as alice_mlstm_step for steps of many tokens a sequence, a chunk at a time on the matrix cores;
-// work: T * (H * dv + H) float32.  Sizes it does not cover (alice_mlstm_chunks_supported) are refused.
+// work: alice_mlstm_chunks_workspace(...) float32; max_new: the most tokens of one sequence in the step.  Sizes it
+// does not cover (alice_mlstm_chunks_supported) are refused.
+extern "C" long alice_mlstm_chunks_workspace(int T, int n_seqs, int max_new, int H, int d, int dv) {
+  int C, VS;
+  chunk_plan(n_seqs, H, d, dv, &C, &VS);
+  long n = (long)T * ((long)H * dv + H);
+  if (C && max_new > C && (long)n_seqs * H * (dv / 16) < 256)           // the chunks side by side: their states too
+    n += 4 + (long)n_seqs * ((max_new + C - 1) / C) * H * ((long)d * dv + d + 3);
+  return n;
+}
+
 extern "C" int alice_mlstm_chunks(const float* proj, int row_w, const float* bias_i, const float* bias_f,
                                   const void* norm_w, int norm_dtype, void* out, int out_dtype, float* work,
                                   const int* cu_seqlens, const int* slots, float* S, float* n, float* m,
                                   int T, int n_seqs, int n_slots, int H, int d, int dv, float cap, float eps,
-                                  hipStream_t stream) {
+                                  int max_new, hipStream_t stream) {
   ALICE_CHECK(dtype_ok(out_dtype) && dtype_ok(norm_dtype), "mlstm: unknown dtype");
   ALICE_CHECK(T >= 0 && n_seqs >= 0 && H >= 1 && H <= 65535 && d >= 1 && dv >= 1, "mlstm: bad sizes H=%d d=%d dv=%d", H, d, dv);
   ALICE_CHECK(row_w >= 2 * H * d + 2 * H * dv + 2 * H && row_w % 4 == 0 && ((uintptr_t)proj & 15) == 0,
               "mlstm: rows of %d numbers are too short, or not a multiple of four numbers from a 16-byte boundary", row_w);
   ALICE_CHECK(proj && bias_i && bias_f && norm_w && out && work && cu_seqlens && slots && S && n && m && n_slots >= 1,
               "mlstm: a pointer is missing");
+  ALICE_CHECK(max_new >= 1 && max_new <= T, "mlstm: the longest piece of the step, %d tokens, is outside 1..%d", max_new, T);
   int C, VS;
   chunk_plan(n_seqs, H, d, dv, &C, &VS);
   ALICE_CHECK(C != 0, "mlstm: the chunk kernel does not cover head sizes %d and %d", d, dv);
   if (n_seqs == 0 || T == 0) return 0;
-  const size_t lds = chunk_lds_bytes(C, VS, d);
   float* dens = work + (size_t)T * H * dv;               // the denominators, [T, H], behind the read-outs
-  dim3 grid(n_seqs, H, dv / VS);
-#define GO(CC, VV)                                                                                                   \
+  const bool side_by_side = max_new > C && (long)n_seqs * H * (dv / 16) < 256;
+  ChunkSpace ws = {nullptr, nullptr, nullptr, nullptr, 1};
+  if (side_by_side) {
+    ws.max_chunks = (max_new + C - 1) / C;
+    const size_t nc = (size_t)n_seqs * ws.max_chunks * H;
+    ws.S = dens + (((size_t)T * H + 3) & ~(size_t)3);          // 16-byte aligned
+    ws.n = ws.S + nc * d * dv;
+    ws.sc = ws.n + nc * d;
+    ws.m0 = ws.sc + nc * 2;
+    chunk_plan(n_seqs * ws.max_chunks, H, d, dv, &C, &VS);          // the slices for that many blocks (C is the same)
+  }
+  const size_t lds = chunk_lds_bytes(C, VS, d);
+#define GO_MODE(CC, VV, MODE, GX)                                                                                    \
   do {                                                                                                               \
     static bool raised = false; /* blocks of more than 64 KB of shared memory: said once per kernel */              \
     if (!raised) {                                                                                                   \
-      hipFuncSetAttribute((const void*)mlstm_chunk_kernel<CC, VV>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+      hipFuncSetAttribute((const void*)mlstm_chunk_kernel<CC, VV, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
       (void)hipGetLastError();                                                                                       \
       raised = true;                                                                                                 \
     }                                                                                                                \
-    mlstm_chunk_kernel<CC, VV><<<grid, CTHREADS, lds, stream>>>(proj, row_w, bias_i, bias_f, work, dens, cu_seqlens, slots, \
-                                                               S, n, m, H, d, dv, cap);                              \
+    mlstm_chunk_kernel<CC, VV, MODE><<<dim3(GX, H, dv / VS), CTHREADS, lds, stream>>>(proj, row_w, bias_i, bias_f, work, dens, \
+        cu_seqlens, slots, S, n, m, H, d, dv, cap, ws);                                                              \
   } while (0)
-  if (C == 64 && VS == 64) GO(64, 64);
-  else if (C == 64 && VS == 32) GO(64, 32);
-  else if (C == 64) GO(64, 16);
-  else if (VS == 32) GO(32, 32);
-  else GO(32, 16);
+#define GO(MODE, GX)                                      \
+  do {                                                    \
+    if (C == 64 && VS == 64) GO_MODE(64, 64, MODE, GX);   \
+    else if (C == 64 && VS == 32) GO_MODE(64, 32, MODE, GX); \
+    else if (C == 64) GO_MODE(64, 16, MODE, GX);          \
+    else if (VS == 32) GO_MODE(32, 32, MODE, GX);         \
+    else GO_MODE(32, 16, MODE, GX);                       \
+  } while (0)
+  if (!side_by_side) {
+    GO(0, n_seqs);
+  } else {
+    GO(1, n_seqs * ws.max_chunks);
+    ALICE_LAUNCH_CHECK();
+    mlstm_chunk_states_kernel<<<dim3(n_seqs, H, ceil_div((long)d * dv / 4, THREADS)), THREADS, 0, stream>>>(
+        cu_seqlens, slots, S, n, m, H, d, dv, C, ws);
+    ALICE_LAUNCH_CHECK();
+    GO(2, n_seqs * ws.max_chunks);
+  }
 #undef GO
+#undef GO_MODE
   ALICE_LAUNCH_CHECK();
   const int threads = dv >= 256 ? 256 : (dv >= 128 ? 128 : 64);
   if (out_dtype == DT_F32)

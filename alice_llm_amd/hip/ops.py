@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib = None
 _lib_path = None
@@ -46,7 +46,7 @@ def _declare(lib) -> None:
         "alice_frag16_supported": [I, I, I],
         "alice_rope_cache_write": [P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, I, I, P],
         "alice_mlstm_step": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, F, F, P],
-        "alice_mlstm_chunks": [P, I, P, P, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
+        "alice_mlstm_chunks": [P, I, P, P, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P],
         "alice_mlstm_chunks_supported": [I, I, I, I],
         "alice_mlstm_cols": [P, I, P, P, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
         "alice_gelu_mul_rows": [P, I, P, I, I, I, P, P, I, I, I, I, I, P],
@@ -69,6 +69,8 @@ def _declare(lib) -> None:
         fn.restype = I
     lib.alice_attention_decode_workspace.argtypes = [I, I, I, I]
     lib.alice_attention_decode_workspace.restype = L
+    lib.alice_mlstm_chunks_workspace.argtypes = [I, I, I, I, I, I]
+    lib.alice_mlstm_chunks_workspace.restype = L
 
 
 def _open(path: str):
@@ -646,7 +648,7 @@ def mlstm_rows(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, *,
     if (max_new >= MLSTM_CHUNK_FROM and proj.shape[1] % 4 == 0
             and library().alice_mlstm_chunks_supported(int(n_seqs), heads, head_dim, value_head_dim)):
         mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
-                     head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps)
+                     head_dim=head_dim, value_head_dim=value_head_dim, cap=cap, eps=eps, max_new=max_new)
         return
     if head_dim <= MLSTM_COLS_MAX_KEY_DIM:
         mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs=n_seqs, heads=heads,
@@ -681,16 +683,26 @@ def _mlstm_args(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n
 
 
 def mlstm_chunks(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, *, n_seqs: int, heads: int, head_dim: int,
-                 value_head_dim: int, cap: float, eps: float, entry: str = "alice_mlstm_chunks") -> None:
+                 value_head_dim: int, cap: float, eps: float, entry: str = "alice_mlstm_chunks",
+                 max_new: Optional[int] = None) -> None:
     """mlstm_step's result by the chunk kernel, or with entry="alice_mlstm_cols" by the kernel of single tokens
     (see mlstm.hip); allocates their float32 workspace [T, H dv]."""
     H, d, dv = heads, head_dim, value_head_dim
     T, n_slots = _mlstm_args(proj, bias_i, bias_f, norm_w, out, cu_seqlens, slots, S, n, m, n_seqs, H, d, dv)
-    work = torch.empty((T, H * dv + H), dtype=torch.float32, device=proj.device)     # read-outs, then denominators
-    _call(entry, proj.data_ptr(), proj.shape[1], bias_i.data_ptr(), bias_f.data_ptr(), norm_w.data_ptr(),
-          dtype_code(norm_w.dtype), out.data_ptr(), dtype_code(out.dtype), work.data_ptr(), cu_seqlens.data_ptr(),
-          slots.data_ptr(), S.data_ptr(), n.data_ptr(), m.data_ptr(), T, int(n_seqs), int(n_slots), H, d, dv, float(cap),
-          float(eps), _stream())
+    args = [proj.data_ptr(), proj.shape[1], bias_i.data_ptr(), bias_f.data_ptr(), norm_w.data_ptr(), dtype_code(norm_w.dtype),
+            out.data_ptr(), dtype_code(out.dtype)]
+    tail = [cu_seqlens.data_ptr(), slots.data_ptr(), S.data_ptr(), n.data_ptr(), m.data_ptr(), T, int(n_seqs), int(n_slots),
+            H, d, dv, float(cap), float(eps)]
+    if entry == "alice_mlstm_chunks":
+        # read-outs, denominators and, where the chunks run side by side, every chunk's state; max_new: the most
+        # tokens of one sequence (the whole step's where the caller does not say)
+        max_new = T if max_new is None else max(1, min(int(max_new), T))
+        work = torch.empty((library().alice_mlstm_chunks_workspace(T, int(n_seqs), max_new, H, d, dv),), dtype=torch.float32,
+                           device=proj.device)
+        _call(entry, *args, work.data_ptr(), *tail, max_new, _stream())
+    else:
+        work = torch.empty((T, H * dv), dtype=torch.float32, device=proj.device)
+        _call(entry, *args, work.data_ptr(), *tail, _stream())
 
 
 def mlstm_step(proj: torch.Tensor, bias_i: torch.Tensor, bias_f: torch.Tensor, norm_w: torch.Tensor, out: torch.Tensor,

@@ -174,6 +174,35 @@ def test_matrix_memory_kernels(dtype, H, d, dv):
     assert torch.all(S[4] == 3.0) and torch.all(S[2] == 0)
 
 
+def test_matrix_memory_chunks_side_by_side_and_one_after_the_other():
+    """A step that leaves the chip unfilled runs its chunks side by side (every chunk's own sums, a walk over the
+    chunks' states, then the read-outs); with max_new below a chunk's length the same rows go through the single
+    pass.  Both against the plain recurrence, and the states they leave against each other."""
+    H, d, dv, cap, eps = 2, 32, 64, 9.0, 1e-5
+    lens = [300, 64, 65, 1]
+    T = sum(lens)
+    x = _mlstm_inputs(T, H, d, dv, seed=21)[:, :2 * H * d + 2 * H * dv + 2 * H].contiguous()   # rows of whole 16-byte units
+    bi, bf, w = rnd(H, seed=1), rnd(H, seed=2) + 2.0, 1 + 0.2 * rnd(H * dv, seed=3)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    slots = torch.tensor([2, 0, 3, 1], dtype=torch.int32, device=DEV)
+    ends = []
+    for max_new in (max(lens), 64):                             # 64: not above a chunk's length, so the single pass
+        S = torch.zeros(4, H, d, dv, device=DEV); n = torch.zeros(4, H, d, device=DEV); m = torch.zeros(4, H, device=DEV)
+        out = torch.empty(T, H * dv, device=DEV)
+        ops.mlstm_chunks(x.to(DEV), bi.to(DEV), bf.to(DEV), w.to(DEV), out, cu, slots, S, n, m, n_seqs=4, heads=H, head_dim=d,
+                         value_head_dim=dv, cap=cap, eps=eps, max_new=max_new)
+        at = 0
+        for b, L in enumerate(lens):
+            ref, st = _mlstm_plain(x[at:at + L], bi, bf, w, H, d, dv, cap, eps)
+            assert max_err(out[at:at + L], ref) < 3e-5 * max(1.0, float(ref.abs().max())), (max_new, b)
+            assert max_err(S[int(slots[b])], st[0]) < 1e-4 * max(1.0, float(st[0].abs().max()))
+            assert max_err(m[int(slots[b])], st[2]) < 1e-4
+            at += L
+        ends.append((S.clone(), n.clone(), m.clone()))
+    for a, b in zip(*ends):
+        assert max_err(a, b) < 1e-4 * max(1.0, float(a.abs().max()))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_matrix_memory_keeps_a_far_token(dtype):
     """One early token is written with a wide-open input gate while every later forget gate stays open: hundreds of
