@@ -18,7 +18,7 @@ from .cache import PAGE_SIZE
 from .engine.generate import MAX_STEP_TOKENS, GenerationResult, Generator
 from .hip import ops
 from .parts import Precision
-from .weights.loader import init_random, load_weights
+from .weights.loader import config_of_folder, init_random, load_weights
 
 
 class Model:
@@ -37,7 +37,7 @@ class Model:
         strict=False: tensors in the folder that the model does not declare are warned about, not an error.
         keep_stored_dtype: on the bfloat16 path, matrices that the folder stores in 32-bit stay 32-bit (and run
         on the plain kernel) instead of being rounded to bfloat16 once at load."""
-        config = load_config(folder)
+        config = config_of_folder(folder)
         device = torch.device(device) if device is not None else ops.require_gpu()
         precision = Precision.of(dtype or getattr(config, "torch_dtype", "bfloat16"), keep_stored_dtype)
         lm = CausalLM(config.plan(), precision, device)

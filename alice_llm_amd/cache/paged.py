@@ -114,7 +114,8 @@ class PageGroup:
         first_needed = max(0, length + 1 - w)        # oldest key of the next query
         tab = self._table[slot]
         changed = False
-        for i in range(min(first_needed // self.page_size, len(tab))):
+        kept = -(-self.need.keep_first // self.page_size)      # pages of the first positions that stay visible
+        for i in range(kept, min(first_needed // self.page_size, len(tab))):
             if tab[i] >= 0:
                 self._free.append(tab[i])
                 tab[i] = -1

@@ -50,10 +50,12 @@ class ScheduleEntry:
     caches, one per run), unless `cache_from` names an earlier entry of the schedule, by its index,
     whose cache this run reads instead of writing one (the reference's kv_layer_map,
     llama3.rs:4739-4745).  `before` names one of the plan's shared parts (a stream operation) that acts on
-    the residual stream right before this run."""
+    the residual stream right before this run; `before_arg`, where given, is handed to that operation (the number
+    of the pass that starts here, for an operation that differs from pass to pass)."""
     layer: int
     cache_from: Optional[int] = None
     before: Optional[str] = None
+    before_arg: Optional[int] = None
 
 
 @dataclass(frozen=True)

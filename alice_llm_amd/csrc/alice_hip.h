@@ -4,12 +4,14 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 8
+#define ALICE_ABI_VERSION 9
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked; epi_param 0: y = gelu_tanh(gate x) * (up x); epi_param = limit > 0:
                               // g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1)
-#define ALICE_EPI_SOFTCAP 2   // y = cap * tanh(y / cap)
+#define ALICE_EPI_SOFTCAP 2   // one function of each output element, its form picked by epi_param: cap > 0: y = cap * tanh(y / cap);
+                              // ALICE_UNARY_RELU2: y = max(y, 0)^2
+#define ALICE_UNARY_RELU2 (-1.0f)
 #define ALICE_EPI_ROPE 3      // internal: rotation and cache write (alice_linear_rope_cache)
 
 #define ALICE_LAYOUT_ROW 0     // row-major [N, K]
@@ -109,6 +111,36 @@ int alice_attention_prefill(const void* q, const void* k_pool, const void* v_poo
                             int bt_stride, int B, int max_new, int nH, int nKV, int d, int page_size,
                             float scale, float softcap, int window, int variant, int out_layout, hipStream_t stream);
 // out[t, h, :] *= sigmoid(gate[t * gate_stride + h]) in place on a bfloat16 attention output in either layout.
+// alice_attention_generic with further parameters of the mask and the softmax (0 / null: off): gate: float32 rows,
+// gate_mode 1: a number a head, 2: a number an output element ([T, nH dv]); out_scale: a constant factor of the
+// gated output; chunk: keys of the query's own chunk of that many
+// positions only; keep_first: the first positions stay visible beside the window; sink [nH]: a term of the
+// softmax's denominator without a value; vrot_cos / vrot_sin [positions, dv / 2]: the head's output is turned back
+// by the query's position; out32 [T, nH, nKV, dv]: every head's weights applied to each kv head's values, float32,
+// nothing written to out (alice_mix_heads follows).
+int alice_attention_masked(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
+                           const int* positions, const int* seq_of_token, const int* block_table,
+                           int bt_stride, int T, int nH, int nKV, int d, int page_size, float scale,
+                           float softcap, int window, const float* bias_slopes, int full_precision,
+                           int dv, const float* gate, int gate_stride, int gate_mode, float out_scale, int chunk,
+                           int keep_first, const float* sink, const float* vrot_cos, const float* vrot_sin,
+                           float* out32, hipStream_t stream);
+// out[t, h, e] = out_scale * sigmoid(gate[t, h dv + e]) * sum_g talk[h, g] a[t, g, kv head of h, e] (gate optional)
+int alice_mix_heads(const float* a, const float* talk, const float* gate, int gate_stride, float out_scale, void* out,
+                    int dtype, int T, int nH, int nKV, int dv, int full_precision, hipStream_t stream);
+// Bias, rotation in pairs (of q, k and optionally v) and the cache write for a fused projection's rows, see qkv_prepare.hip.
+int alice_qkv_prepare(const void* rows, int rows_dtype, int row_width, const float* bias, void* q_out, void* k_pool,
+                      void* v_pool, int out_dtype, const float* cos_t, const float* sin_t, int rotary_dim,
+                      int interleaved, const float* vcos, const float* vsin, const int* positions,
+                      const int* seq_of_token, const int* block_table, int bt_stride, int T, int nH, int nKV,
+                      int d, int dv, int page_size, int n_pages, hipStream_t stream);
+// x[t, c] += a[t, c] + v[c] (either may be null)
+int alice_add_rows(float* x, const float* a, const float* v, int T, int W, hipStream_t stream);
+// Gated linear attention over a step's tokens, see gla.hip.
+int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, const float* z,
+              const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
+              int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
+              int n_slots, int H, int d, int dv, hipStream_t stream);
 int alice_head_gate(void* out, int out_layout, const void* gate, int gate_stride, int T, int nH, int d, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 // out may be absent when splits > 1: the splits are then left in `parts`, [B][nH][splits][ALICE_ATTN_PARTS_HEAD + d]

@@ -114,6 +114,15 @@ __device__ __forceinline__ float gated_act(float g, float u, float limit, bool f
   }
   return gelu_tanh_f(g, full) * u;
 }
+// The function of one output element, the epilogue ALICE_EPI_SOFTCAP.  Its parameter picks the form: a positive cap
+// gives cap * tanh(v / cap); a negative one (ALICE_UNARY_RELU2) the square of max(v, 0).
+__device__ __forceinline__ float unary_act(float v, float p, bool full) {
+  if (p < 0.f) {
+    const float r = fmaxf(v, 0.f);
+    return r * r;
+  }
+  return p * (full ? tanh_full(v / p) : tanh_fast(v / p));
+}
 __device__ __forceinline__ float sigmoid_f(float z, bool full) { return 1.f / (1.f + (full ? expf(-z) : __expf(-z))); }
 
 // ---- host side -------------------------------------------------------------------------

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void linear_tiled_kernel(const TA* __restrict_
         const int n = (j < 2 ? n0 : n1) + tx * 2 + (j & 1);
         if (n < N) {
           float v = acc[i][j];
-          if (EPI == ALICE_EPI_SOFTCAP) v = epi * (FULL ? tanh_full(v / epi) : tanh_fast(v / epi));
+          if (EPI == ALICE_EPI_SOFTCAP) v = unary_act(v, epi, FULL);
           store_f32(Y, (size_t)m * N + n, v);
         }
       }
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(const TA* __restrict__
     if (lane == 0) {
       float o = v[0];
       if (EPI == ALICE_EPI_GEGLU) o = gated_act(v[0], v[NR - 1], epi, FULL);
-      if (EPI == ALICE_EPI_SOFTCAP) o = epi * (FULL ? tanh_full(o / epi) : tanh_fast(o / epi));
+      if (EPI == ALICE_EPI_SOFTCAP) o = unary_act(o, epi, FULL);
       store_f32(Y, (size_t)m * N + n, o);
     }
   }
@@ -193,7 +193,7 @@ int alice_linear_generic(const void* x, int x_dtype, const void* w, int w_dtype,
   ALICE_CHECK(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   ALICE_CHECK(epi == ALICE_EPI_NONE || epi == ALICE_EPI_GEGLU || epi == ALICE_EPI_SOFTCAP,
               "linear: unknown epilogue %d", epi);
-  ALICE_CHECK(epi != ALICE_EPI_SOFTCAP || epi_param > 0.f, "linear: softcap must be positive");
+  ALICE_CHECK(epi != ALICE_EPI_SOFTCAP || epi_param > 0.f || epi_param == ALICE_UNARY_RELU2, "linear: softcap must be positive");
   ALICE_CHECK(ceil_div(M, BM) <= 65535, "linear: M=%d has too many row tiles for one launch", M);
   if (M == 0) return 0;
   int rc = 0;

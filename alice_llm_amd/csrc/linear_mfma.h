@@ -73,7 +73,7 @@ __device__ __forceinline__ u32x4 load_x_frag_f(const bf16_t* __restrict__ x, int
 
 template <int EPI, bool FULL>
 __device__ __forceinline__ float epilogue1(float v, float p) {
-  if (EPI == ALICE_EPI_SOFTCAP) return p * (FULL ? tanh_full(v / p) : tanh_fast(v / p));
+  if (EPI == ALICE_EPI_SOFTCAP) return unary_act(v, p, FULL);
   return v;
 }
 

@@ -76,7 +76,7 @@ int alice_linear_frag(const void* x, int x_dtype, const void* w, void* y, int y_
   ALICE_CHECK(dtype_ok(y_dtype), "linear: unknown output dtype");
   ALICE_CHECK(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear: bad sizes M=%d N=%d K=%d (K must be a multiple of 8)", M, N, K);
   ALICE_CHECK(epi != ALICE_EPI_GEGLU || N % 16 == 0, "linear: GeGLU in the fragment layout needs N %% 16 == 0, found %d", N);
-  ALICE_CHECK(epi != ALICE_EPI_SOFTCAP || epi_param > 0.f, "linear: softcap must be positive");
+  ALICE_CHECK(epi != ALICE_EPI_SOFTCAP || epi_param > 0.f || epi_param == ALICE_UNARY_RELU2, "linear: softcap must be positive");
   ALICE_CHECK(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0, "linear: operands must be 16-byte aligned");
   ALICE_CHECK(x_layout == ALICE_LAYOUT_ROW || (x_layout == ALICE_LAYOUT_FRAG16 && K % 32 == 0),
               "linear: activations in fragment order need K %% 32 == 0, found K=%d", K);

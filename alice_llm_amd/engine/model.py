@@ -164,7 +164,10 @@ class CausalLM:
             stream.start = stream.x.clone()            # the embedding output, for stream operations that read it
         for i, entry in enumerate(self.plan.schedule):
             if entry.before is not None:
-                self.shared[entry.before].apply(stream, ctx)
+                if entry.before_arg is None:
+                    self.shared[entry.before].apply(stream, ctx)
+                else:
+                    self.shared[entry.before].apply(stream, ctx, entry.before_arg)
             view = cache.view(i, block_tables, read_from=entry.cache_from)
             self.layers[entry.layer].block.forward(stream, ctx, view)
         if ctx.want_rows is None or ctx.want_rows.numel() == 0:

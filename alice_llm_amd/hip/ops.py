@@ -18,7 +18,8 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 8
+ABI_VERSION = 9
+UNARY_RELU2 = -1.0       # epi_param of EPI_SOFTCAP that picks the square of max(y, 0) instead of the capped form
 
 _lib = None
 _lib_path = None
@@ -56,6 +57,11 @@ def _declare(lib) -> None:
         "alice_attention_decode": [P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, I, I, P, I, P],
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, P],
         "alice_head_gate": [P, I, P, I, I, I, I, P],
+        "alice_attention_masked": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, I, F, I, I, P, P, P, P, P],
+        "alice_mix_heads": [P, P, P, I, F, P, I, I, I, I, I, I, P],
+        "alice_qkv_prepare": [P, I, I, P, P, P, P, I, P, P, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "alice_add_rows": [P, P, P, I, I, P],
+        "alice_gla": [P, I, I, I, I, I, P, P, F, F, F, P, I, F, P, I, P, P, P, P, I, I, I, I, I, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
@@ -460,6 +466,179 @@ def attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
           block_table.shape[1], T, num_heads, nKV, d, page_size, float(scale),
           float(softcap or 0.0), int(window or 0), None if bias_slopes is None else bias_slopes.data_ptr(),
           int(full_precision), int(dv), gate_ptr, int(gate_stride), _stream())
+
+
+def attention_masked(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: Optional[torch.Tensor],
+                     positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, *,
+                     num_heads: int, scale: float, max_position: int, full_precision: bool,
+                     softcap: Optional[float] = None, window: Optional[int] = None, chunk: Optional[int] = None,
+                     keep_first: int = 0, bias_slopes: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+                     gate: Optional[torch.Tensor] = None, gate_per_element: bool = False, out_scale: float = 1.0,
+                     value_cos: Optional[torch.Tensor] = None, value_sin: Optional[torch.Tensor] = None,
+                     per_value_head: Optional[torch.Tensor] = None) -> None:
+    """attention_generic with further masks and softmax terms over a row-major cache.  chunk: a query sees the keys
+    of its own chunk of that many positions (counted from position 0); keep_first: keys below that position stay
+    visible beside the window; sink: float32 [heads], a term of the denominator without a value; gate: float32
+    [T, >= heads] (rows of any stride), with gate_per_element [T, >= heads * dv], one number an output element;
+    out_scale: a constant factor of the gated output; value_cos / value_sin: float32
+    [positions, dv / 2], the output of a head is turned back by the query's position (the values were cached turned
+    by their own); per_value_head: float32 [T, heads, kv heads, dv] that receives every head's weights applied to
+    each kv head's values (nothing goes to out, and no gate is applied: mix_heads follows)."""
+    T = q.shape[0]
+    dt = q.dtype
+    if k_pool.dim() != 4 or v_pool.dim() != 4:
+        raise HipLibraryError("k_pool must be [pages, nKV, page, d]")
+    n_pages, nKV, page_size, d = k_pool.shape
+    dv = v_pool.shape[3]
+    _dev(q, "q", None, (T, num_heads * d))
+    _dev(k_pool, "k_pool", dt)
+    _dev(v_pool, "v_pool", dt, tuple(k_pool.shape[:3]) + (dv,))
+    if per_value_head is not None:
+        _dev(per_value_head, "per_value_head", torch.float32, (T, num_heads, nKV, dv))
+        if gate is not None:
+            raise HipLibraryError("per-value-head outputs take no gate: the mix that follows does")
+    else:
+        _dev(out, "out", dt, (T, num_heads * dv))
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        need = num_heads * dv if gate_per_element else num_heads
+        if (not gate.is_cuda or gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < need
+                or gate.stride(1) != 1 or gate.stride(0) < need):
+            raise HipLibraryError(f"gate must be [{T}, >= {need}] float32 with unit column stride")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
+    _dev(positions, "positions", torch.int32, (T,))
+    _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
+    _dev(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
+        raise HipLibraryError(f"position {max_position} is beyond the block table {tuple(block_table.shape)}")
+    if bias_slopes is not None:
+        _dev(bias_slopes, "bias_slopes", torch.float32, (num_heads,))
+    if sink is not None:
+        _dev(sink, "sink", torch.float32, (num_heads,))
+    if value_cos is not None:
+        if dv % 2 or value_cos.dim() != 2 or value_cos.shape[1] != dv // 2 or value_sin.shape != value_cos.shape:
+            raise HipLibraryError(f"value tables must be [positions, {dv // 2}]")
+        _dev(value_cos, "value_cos", torch.float32)
+        _dev(value_sin, "value_sin", torch.float32)
+        if max_position >= value_cos.shape[0]:
+            raise HipLibraryError(f"position {max_position} is beyond the rotation tables ({value_cos.shape[0]} positions)")
+    _call("alice_attention_masked", q.data_ptr(), dtype_code(dt), k_pool.data_ptr(), v_pool.data_ptr(),
+          None if out is None else out.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+          block_table.shape[1], T, num_heads, nKV, d, page_size, float(scale), float(softcap or 0.0), int(window or 0),
+          None if bias_slopes is None else bias_slopes.data_ptr(), int(full_precision), int(dv), gate_ptr, int(gate_stride),
+          2 if gate_per_element else 1, float(out_scale), int(chunk or 0), int(keep_first or 0), None if sink is None else sink.data_ptr(),
+          None if value_cos is None else value_cos.data_ptr(), None if value_sin is None else value_sin.data_ptr(),
+          None if per_value_head is None else per_value_head.data_ptr(), _stream())
+
+
+def mix_heads(a: torch.Tensor, talk: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, *,
+              full_precision: bool, out_scale: float = 1.0) -> None:
+    """out[t, h, :] = out_scale * sigmoid(gate[t, h, :]) * sum_g talk[h, g] * a[t, g, kv head of h, :]; a: float32
+    [T, heads, kv heads, dv]; talk: float32 [heads, heads]; gate: float32 [T, >= heads * dv] (or None)."""
+    if a.dim() != 4:
+        raise HipLibraryError("a must be [T, heads, kv heads, dv]")
+    T, H, G, dv = a.shape
+    _dev(a, "a", torch.float32)
+    _dev(talk, "talk", torch.float32, (H, H))
+    _dev(out, "out", None, (T, H * dv))
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        if (not gate.is_cuda or gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < H * dv
+                or gate.stride(1) != 1):
+            raise HipLibraryError(f"gate must be [{T}, >= {H * dv}] float32 with unit column stride")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
+    _call("alice_mix_heads", a.data_ptr(), talk.data_ptr(), gate_ptr, int(gate_stride), float(out_scale), out.data_ptr(),
+          dtype_code(out.dtype), T, H, G, dv, int(full_precision), _stream())
+
+
+def qkv_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.Tensor, k_pool: Optional[torch.Tensor],
+                v_pool: Optional[torch.Tensor], positions: torch.Tensor, seq_of_token: Optional[torch.Tensor],
+                block_table: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int, head_dim: int,
+                value_head_dim: int, max_position: int, cos: Optional[torch.Tensor] = None,
+                sin: Optional[torch.Tensor] = None, rotary_dim: int = 0, interleaved: bool = True,
+                value_cos: Optional[torch.Tensor] = None, value_sin: Optional[torch.Tensor] = None) -> None:
+    """From the rows [q | k | v | ...] of a fused projection (float32, or q_out's dtype): bias [>= q, k, v columns]
+    added, q and k heads rotated over their first rotary_dim dimensions in pairs ((2i, 2i + 1) if interleaved, else
+    (i, i + rotary_dim / 2)) from tables [positions, rotary_dim / 2], values turned over all their dimensions where
+    value tables [positions, dv / 2] are given; q to q_out, k and v into the row-major pools at their positions."""
+    T = rows.shape[0]
+    dt = q_out.dtype
+    d, dv = head_dim, value_head_dim
+    if rows.dim() != 2 or rows.dtype not in (torch.float32, dt):
+        raise HipLibraryError("rows must be [T, width] in float32 or the outputs' dtype")
+    _dev(rows, "rows")
+    width = num_heads * d + (num_kv_heads * (d + dv) if k_pool is not None else 0)
+    if rows.shape[1] < width:
+        raise HipLibraryError(f"rows of {tuple(rows.shape)} are too short for the heads")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() < width:
+            raise HipLibraryError(f"bias must hold {width} elements")
+    _dev(q_out, "q_out", None, (T, num_heads * d))
+    _dev(positions, "positions", torch.int32, (T,))
+    for c, s_, n, what in ((cos, sin, rotary_dim, "cos/sin"), (value_cos, value_sin, dv, "value tables")):
+        if c is not None:
+            if c.dim() != 2 or c.shape[1] != n // 2 or s_.shape != c.shape or n % 2:
+                raise HipLibraryError(f"{what} must be [positions, {n // 2}]")
+            _dev(c, what, torch.float32)
+            _dev(s_, what, torch.float32)
+            if max_position >= c.shape[0]:
+                raise HipLibraryError(f"position {max_position} is beyond the rotation tables ({c.shape[0]} positions)")
+    page_size = n_pages = bt_stride = 0
+    if k_pool is not None:
+        if k_pool.dim() != 4 or k_pool.shape[1] != num_kv_heads or k_pool.shape[3] != d:
+            raise HipLibraryError(f"k_pool must be [pages, {num_kv_heads}, page, {d}], found {tuple(k_pool.shape)}")
+        _dev(k_pool, "k_pool", dt)
+        _dev(v_pool, "v_pool", dt, tuple(k_pool.shape[:3]) + (dv,))
+        n_pages, _, page_size, _ = k_pool.shape
+        _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
+        _dev(block_table, "block_table", torch.int32)
+        if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
+            raise HipLibraryError(f"position {max_position} is beyond the block table")
+        bt_stride = block_table.shape[1]
+    _call("alice_qkv_prepare", rows.data_ptr(), dtype_code(rows.dtype), rows.shape[1], _opt(bias, "bias"), q_out.data_ptr(),
+          _opt(k_pool, "k_pool"), _opt(v_pool, "v_pool"), dtype_code(dt), _opt(cos, "cos"), _opt(sin, "sin"),
+          int(rotary_dim if cos is not None else 0), int(interleaved), _opt(value_cos, "value_cos"), _opt(value_sin, "value_sin"),
+          positions.data_ptr(), _opt(seq_of_token, "seq_of_token"), _opt(block_table, "block_table"), bt_stride, T,
+          num_heads, num_kv_heads if k_pool is not None else 0, d, dv, page_size, n_pages, _stream())
+
+
+def add_rows(x: torch.Tensor, rows: Optional[torch.Tensor], vector: Optional[torch.Tensor]) -> None:
+    """x[t, :] += rows[t, :] + vector (either may be None); all float32."""
+    T, W = x.shape
+    _dev(x, "x", torch.float32)
+    _call("alice_add_rows", x.data_ptr(), _opt(rows, "rows", torch.float32, (T, W)), _opt(vector, "vector", torch.float32, (W,)),
+          T, W, _stream())
+
+
+GLA_MAX_KEY_DIM = 256       # the largest key size the gated linear attention kernel keeps in registers
+
+
+def gla(rows: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, norm_w: torch.Tensor, out: torch.Tensor, ctx,
+        S: torch.Tensor, *, heads: int, head_dim: int, value_head_dim: int, tau: float, q_scale: float, eps: float,
+        columns, out_scale: float = 1.0) -> None:
+    """Gated linear attention over a step (`ctx` gives cu_seqlens, slots, n_seqs): rows float32 [T, width] with q, k,
+    v and the gate at `columns` = (q, k, v, g); z float32 [T, heads * d] and z_bias float32 [heads * d]: the decay is
+    sigmoid(z + z_bias)^(1 / tau); S float32 [slots, heads, d, dv]; out [T, heads * dv], times out_scale."""
+    H, d, dv = heads, head_dim, value_head_dim
+    T = rows.shape[0]
+    _dev(rows, "rows", torch.float32)
+    _dev(z, "z", torch.float32, (T, H * d))
+    _dev(z_bias, "z_bias", torch.float32, (H * d,))
+    _dev(norm_w, "norm_w", None, (dv,))
+    _dev(out, "out", None, (T, H * dv))
+    _dev(ctx.cu_seqlens, "cu_seqlens", torch.int32)
+    _dev(ctx.slots, "slots", torch.int32)
+    if ctx.cu_seqlens.numel() < ctx.n_seqs + 1 or ctx.slots.numel() < ctx.n_seqs:
+        raise HipLibraryError("cu_seqlens and slots are too short for the step's sequences")
+    n_slots = S.shape[0]
+    _dev(S, "S", torch.float32, (n_slots, H, d, dv))
+    work = torch.empty((T, H * dv), dtype=torch.float32, device=rows.device) if dv > 64 else None
+    q_col, k_col, v_col, g_col = (int(c) for c in columns)
+    _call("alice_gla", rows.data_ptr(), rows.shape[1], q_col, k_col, v_col, g_col, z.data_ptr(), z_bias.data_ptr(), float(tau),
+          float(q_scale), float(out_scale), norm_w.data_ptr(), dtype_code(norm_w.dtype), float(eps), out.data_ptr(), dtype_code(out.dtype),
+          _opt(work, "work"), ctx.cu_seqlens.data_ptr(), ctx.slots.data_ptr(), S.data_ptr(), T, int(ctx.n_seqs), int(n_slots),
+          H, d, dv, _stream())
 
 
 def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:

@@ -12,6 +12,23 @@ in both dtypes).  Values may have a head size of their own (value_head_dim), and
 one gate number a query head, projected from the mixer's input beside q, k and v: head h's output is
 multiplied by sigmoid(gate_h) before the output projection.  tensor_names gives the local names of the
 matrices (q, k, v, o, g) where a file names them otherwise.
+
+Further constructor arguments, each off by default, make other attention mixers from the same part (they run
+on the 32-bit attention kernel over a row-major cache in both dtypes, from a projection whose sums stay 32-bit
+until the bias is added and the rotation done):
+  bias            q, k and v have biases (the matrix's name + ".b"), added in the projection
+  chunk           a query sees the keys of its own chunk of that many positions only, chunks counted from the
+                  sequence's position 0 (the cache gives the pages of finished chunks back like a window's)
+  keep_first      beside its window a query sees the first that many positions (the cache keeps their pages)
+  sink            one learned number a head ("sink") whose exponential joins the softmax's denominator; it has no
+                  key and no value
+  talk            the heads' softmax weights are mixed by a learned matrix ("talk" [heads, heads]) before they meet
+                  the values: weight_h <- sum_g talk[h, g] weight_g, head h keeping its own kv head's values
+  output_gate     "elementwise": sigmoid of a projection of the mixer's input ("g" [heads * value size, width]) times
+                  the concatenated heads
+  output_scale    a constant factor of the mixer's output (applied to the gated heads; the output matrix is linear)
+  position        a "rope_pairs" encoding: pairs of neighbouring dimensions, a rotated part of the head, and
+                  values that are turned by their position and turned back at the output
 """
 from __future__ import annotations
 
@@ -32,7 +49,9 @@ class Attention(Part):
                  num_kv_heads: int, head_dim: int, scale: float, softcap: Optional[float] = None,
                  window: Optional[int] = None, position: Optional[str] = None,
                  score_bias_slopes: Optional[Sequence[float]] = None, value_head_dim: Optional[int] = None,
-                 output_gate: Optional[str] = None, tensor_names: Optional[Dict[str, str]] = None):
+                 output_gate: Optional[str] = None, tensor_names: Optional[Dict[str, str]] = None,
+                 bias: bool = False, chunk: Optional[int] = None, keep_first: int = 0, sink: bool = False,
+                 talk: bool = False, output_scale: float = 1.0):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_kv_heads {num_kv_heads} must divide num_heads {num_heads}")
         if not 1 <= head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
@@ -54,12 +73,29 @@ class Attention(Part):
         self.dv = head_dim if value_head_dim is None else int(value_head_dim)
         if not 1 <= self.dv <= ops.ATTENTION_MAX_HEAD_DIM:
             raise ValueError(f"attention: value_head_dim {self.dv} is outside 1..{ops.ATTENTION_MAX_HEAD_DIM}")
-        if output_gate not in (None, "head"):
-            raise ValueError(f"attention: output_gate '{output_gate}' is not known (None or 'head')")
+        if output_gate not in (None, "head", "elementwise"):
+            raise ValueError(f"attention: output_gate '{output_gate}' is not known (None, 'head' or 'elementwise')")
+        if chunk is not None and (window is not None or chunk < 1):
+            raise ValueError("attention: a chunk is at least 1 position and stands in the window's place")
+        if keep_first < 0 or (keep_first and window is None):
+            raise ValueError("attention: kept first positions go with a window")
         self.output_gate = output_gate
-        self.n_gate = num_heads if output_gate == "head" else 0
+        self.n_gate = {None: 0, "head": num_heads, "elementwise": num_heads * self.dv}[output_gate]
+        self.bias, self.chunk, self.keep_first = bool(bias), chunk, int(keep_first)
+        self.has_sink, self.has_talk, self.output_scale = bool(sink), bool(talk), float(output_scale)
+        pairs = getattr(self.position, "value_cos", "absent") != "absent"          # a rope_pairs encoding
+        # the mixers made by the further arguments: float32 projection sums, bias and rotation in one kernel, the
+        # 32-bit attention kernel with its further masks over a row-major cache
+        self.extended = bool(bias or chunk or keep_first or sink or talk or output_gate == "elementwise"
+                             or output_scale != 1.0 or pairs)
+        if self.extended and softcap is not None and talk:
+            raise ValueError("attention: mixed heads take no softcap")
         self.names = dict({"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-                           "g": "g_proj.weight"}, **(tensor_names or {}))
+                           "g": "g_proj.weight", "sink": "sink", "talk": "talk"}, **(tensor_names or {}))
+        self._bias_parts: Dict[str, torch.Tensor] = {}
+        self.qkv_bias: Optional[torch.Tensor] = None
+        self.sink: Optional[torch.Tensor] = None
+        self.talk: Optional[torch.Tensor] = None
         self.q_dim, self.kv_dim, self.v_dim = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * self.dv
         self.o_in = num_heads * self.dv
         # one fused projection: all q heads, the k heads, the v heads, then the gate numbers
@@ -70,7 +106,7 @@ class Attention(Part):
         # that a run that reads another run's cache finds the layout it expects.
         self.kv_layout = (ops.KV_FRAGMENT if precision.name == "bfloat16" and precision.act == torch.bfloat16
                           and ops.library_ready() and ops.attention_mfma_supported(head_dim)
-                          and score_bias_slopes is None and self.dv == head_dim else ops.KV_ROW)
+                          and score_bias_slopes is None and self.dv == head_dim and not self.extended else ops.KV_ROW)
         self._parts: Dict[str, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -81,19 +117,34 @@ class Attention(Part):
                  n["o"]: ParamSpec((self.H, self.o_in))}
         if self.n_gate:
             specs[n["g"]] = ParamSpec((self.n_gate, self.H))
+        if self.bias:
+            specs[n["q"] + ".b"] = ParamSpec((self.q_dim,), init_std=0.1)
+            specs[n["k"] + ".b"] = ParamSpec((self.kv_dim,), init_std=0.1)
+            specs[n["v"] + ".b"] = ParamSpec((self.v_dim,), init_std=0.1)
+        if self.has_sink:
+            specs[n["sink"]] = ParamSpec((self.nH,), init_std=1.0)
+        if self.has_talk:
+            specs[n["talk"]] = ParamSpec((self.nH, self.nH), init_std=0.3)
         return specs
 
     def cache_need(self) -> CacheNeed:
         # the fragment layout of the matrix-core kernels is written for pages of 64 positions
         page = ops.KV_FRAGMENT_PAGE if self.kv_layout == ops.KV_FRAGMENT else None
-        return CacheNeed(kv=KVNeed(self.nKV, self.d, self.window, page_size=page,
-                                   value_head_dim=None if self.dv == self.d else self.dv))
+        # a chunk's keys lie at most chunk - 1 positions back: its pages go back to the pool like a window's
+        return CacheNeed(kv=KVNeed(self.nKV, self.d, self.window if self.chunk is None else self.chunk, page_size=page,
+                                   value_head_dim=None if self.dv == self.d else self.dv, keep_first=self.keep_first))
 
     def assign(self, name: str, tensor: torch.Tensor) -> None:
         if name == self.names["o"]:
             self.o.load(tensor)
         elif name in [self.names[c] for c in ("qkvg" if self.n_gate else "qkv")]:
             self._parts[name] = tensor
+        elif self.bias and name in [self.names[c] + ".b" for c in "qkv"]:
+            self._bias_parts[name] = tensor
+        elif self.has_sink and name == self.names["sink"]:
+            self.sink = tensor.float().contiguous()
+        elif self.has_talk and name == self.names["talk"]:
+            self.talk = tensor.float().contiguous()
         else:
             raise KeyError(name)
 
@@ -105,7 +156,9 @@ class Attention(Part):
         # a position encoding may ask for the rows of the q and k heads in another order (rotated pairs next to
         # each other), so that its rotation can be the projection's epilogue
         order = getattr(self.position, "projection_row_order", lambda *a: None)(self.nH, self.nKV, self.d)
-        self.pair_order = order is not None and self.dv == self.d and not self.n_gate
+        self.pair_order = order is not None and self.dv == self.d and not self.n_gate and not self.extended
+        if self.bias:
+            self.qkv_bias = torch.cat([self._bias_parts.pop(self.names[c] + ".b").float() for c in "qkv"]).contiguous()
         if self.pair_order:
             w = w[order.to(w.device)]
         self.qkv.load(w)
@@ -123,6 +176,8 @@ class Attention(Part):
         """x: [T, H] in the activation dtype (a tensor, or FragmentActs in decode steps); returns the branch
         in float32 ([T, H] or partial sums)."""
         T = x.shape[0]
+        if self.extended:
+            return self._forward_extended(x, ctx, cache)
         q = torch.empty((T, self.q_dim), dtype=self.precision.act, device=x.device)
         geometry = dict(num_heads=self.nH, num_kv_heads=self.nKV, head_dim=self.d, kv_layout=self.kv_layout)
         if self.dv != self.d:
@@ -160,4 +215,39 @@ class Attention(Part):
                       scale=self.scale, softcap=self.softcap, window=self.window, full_precision=self.precision.full,
                       kv_layout=self.kv_layout, out_layout=ops.LAYOUT_FRAG16 if frag else ops.LAYOUT_ROW,
                       bias_slopes=self._slopes, gate=gate)
+        return self.o(out, torch.float32, allow_partials=True)
+
+    def _forward_extended(self, x, ctx, cache) -> torch.Tensor:
+        """The mixers made by the further constructor arguments (see the top of the file)."""
+        T, act, dev = x.shape[0], self.precision.act, x.device
+        rows = self.qkv(x, torch.float32)                     # [q | k | v | g], the sums as they are
+        q = torch.empty((T, self.q_dim), dtype=act, device=dev)
+        pos = self.position
+        write = cache is not None and cache.writable
+        ops.qkv_prepare(rows, self.qkv_bias, q, cache.k if write else None, cache.v if write else None, ctx.positions,
+                        ctx.seq_of_token if write else None, cache.block_table if write else None,
+                        num_heads=self.nH, num_kv_heads=self.nKV, head_dim=self.d, value_head_dim=self.dv,
+                        max_position=ctx.max_position, cos=getattr(pos, "cos", None), sin=getattr(pos, "sin", None),
+                        rotary_dim=getattr(pos, "rotary_dim", 0), interleaved=getattr(pos, "interleaved", True),
+                        value_cos=getattr(pos, "value_cos", None), value_sin=getattr(pos, "value_sin", None))
+        gate = None
+        if self.n_gate:
+            g0 = self.q_dim + self.kv_dim + self.v_dim
+            gate = rows[:, g0:g0 + self.n_gate]
+        out = torch.empty((T, self.o_in), dtype=act, device=dev)
+        common = dict(num_heads=self.nH, scale=self.scale, softcap=self.softcap, window=self.window, chunk=self.chunk,
+                      keep_first=self.keep_first, max_position=ctx.max_position, full_precision=self.precision.full,
+                      bias_slopes=self._slopes, sink=self.sink, value_cos=getattr(pos, "value_cos", None),
+                      value_sin=getattr(pos, "value_sin", None))
+        if self.has_talk:
+            # every head's weights on each kv head's values, then the mix of the heads with the gate behind it
+            per = torch.empty((T, self.nH, self.nKV, self.dv), dtype=torch.float32, device=dev)
+            ops.attention_masked(q, cache.k, cache.v, None, ctx.positions, ctx.seq_of_token, cache.block_table,
+                                 per_value_head=per, **common)
+            if self.output_gate == "head":
+                raise NotImplementedError("attention: mixed heads take an elementwise gate or none")
+            ops.mix_heads(per, self.talk, gate, out, full_precision=self.precision.full, out_scale=self.output_scale)
+        else:
+            ops.attention_masked(q, cache.k, cache.v, out, ctx.positions, ctx.seq_of_token, cache.block_table, gate=gate,
+                                 gate_per_element=self.output_gate == "elementwise", out_scale=self.output_scale, **common)
         return self.o(out, torch.float32, allow_partials=True)

@@ -116,13 +116,16 @@ class KVNeed:
     (None: all of them).  `page_size`: the number of positions per page that the mixer's kernels are written
     for (None: any); a cache built with another page size refuses the mixer when the model is put together.
     `dtype`: the dtype of the pages (None: the run's activation dtype); a mixer that wants its keys in 32-bit
-    under bfloat16 activations says so here, and its layers get storage of their own."""
+    under bfloat16 activations says so here, and its layers get storage of their own.
+    `keep_first`: with a window, the first that many positions are read by every later query too: their pages
+    are never given back while the sequence lives."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_head_dim: Optional[int] = None
     page_size: Optional[int] = None
     dtype: Optional[torch.dtype] = None
+    keep_first: int = 0
 
     @property
     def v_dim(self) -> int:

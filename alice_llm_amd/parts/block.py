@@ -2,7 +2,8 @@
 
 "sandwich": x += post_mixer(mixer(pre_mixer(x))); x += post_ff(ff(pre_ff(x))), each norm optional
 (llama3.rs:14178, 14460-14470, 14497, 14543-14557: Gemma 2 has all four; a pre-norm-only layer
-leaves the post norms out and is the same wiring).
+leaves the post norms out and is the same wiring).  The feed-forward may be absent, and a mixer may return
+several branches, each with a post norm of its own, which are all added before the feed-forward's norm.
 
 "parallel": one norm, whose output feeds the mixer and the feed-forward side by side:
 h = pre(x); x += mixer(h) + ff(h) (the feed-forward may be absent); then the layer's extras act on the
@@ -20,7 +21,9 @@ from .base import BLOCKS
 class SandwichBlock:
     graph_safe = True
 
-    def __init__(self, mixer, feed_forward, norms: Dict[str, object]):
+    def __init__(self, mixer, feed_forward, norms: Dict[str, object], extras: Dict[str, object] = None):
+        if extras:
+            raise ValueError("the sandwich arrangement has no place for further parts of a layer")
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norms = norms
@@ -30,7 +33,13 @@ class SandwichBlock:
         frag = getattr(ctx, "fragment_activations", False)
         h = stream.normed(self.norms.get("pre_mixer"),
                           fragments=frag and getattr(self.mixer, "accepts_fragment_activations", False))
-        stream.push(self.mixer.forward(h, ctx, cache), self.norms.get("post_mixer"))
+        branches = self.mixer.forward(h, ctx, cache)
+        if isinstance(branches, list):
+            stream.push_many([(b, post if post is not None else self.norms.get("post_mixer")) for b, post in branches])
+        else:
+            stream.push(branches, self.norms.get("post_mixer"))
+        if self.feed_forward is None:
+            return
         h = stream.normed(self.norms.get("pre_ff"),
                           fragments=frag and getattr(self.feed_forward, "accepts_fragment_activations", False))
         stream.push(self.feed_forward.forward(h, ctx), self.norms.get("post_ff"))

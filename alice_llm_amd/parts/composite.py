@@ -5,6 +5,9 @@ output is RMS-normed over the model width with a plain weight of its own (`<side
 the normed outputs are averaged.  The average is folded into the norm weights (w / sides), so every side
 reaches the residual stream as one more branch with its post norm, through the stream's fused add + norm.
 
+With `side_norms=False` the sides' outputs are added as they are (a side that takes a constant factor of its
+output has it among its own constructor arguments), and no norm tensors are declared.
+
 At most one side may keep keys and values in pages; state tensors of the sides are kept apart by the side's
 name.  A part that returns several branches returns a list of (branch, post norm) pairs; blocks push them
 one after the other.
@@ -29,7 +32,7 @@ class _SideCache:
 @MIXERS.register("side_by_side")
 class SideBySide(Part):
     def __init__(self, precision: Precision, positions: dict, *, hidden_size: int, sides: Sequence, norm_eps: float,
-                 norm_tensor: str = "out"):
+                 norm_tensor: str = "out", side_norms: bool = True):
         if not sides:
             raise ValueError("side_by_side needs at least one side")
         self.precision = precision
@@ -40,7 +43,7 @@ class SideBySide(Part):
         self.norm_tensor = norm_tensor
         # the plain-weight RMS norm of each side's output; its weight is kept divided by the number of sides
         self.norms = [NORMS.get("rmsnorm")(precision, dim=hidden_size, eps=norm_eps, weight_offset=0.0,
-                                           tensor_name=norm_tensor) for _ in sides]
+                                           tensor_name=norm_tensor) if side_norms else None for _ in sides]
         needs = [m.cache_need() if hasattr(m, "cache_need") else None for m in self.sides]
         if sum(1 for n in needs if n is not None and n.kv is not None) > 1:
             raise ValueError("side_by_side: only one side may keep keys and values in pages")
@@ -57,7 +60,7 @@ class SideBySide(Part):
 
     @property
     def accepts_fragment_activations(self) -> bool:
-        return False
+        return all(getattr(m, "accepts_fragment_activations", False) for m in self.sides)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         specs: Dict[str, ParamSpec] = {}
@@ -65,7 +68,7 @@ class SideBySide(Part):
             for local, spec in m.param_specs().items():
                 specs[f"{name}.{local}"] = spec
         for name, n in zip(self.names, self.norms):
-            for local, spec in n.param_specs().items():
+            for local, spec in (n.param_specs().items() if n is not None else ()):
                 specs[f"{name}.{local}"] = spec
         return specs
 
@@ -73,7 +76,7 @@ class SideBySide(Part):
         for side, m, n in zip(self.names, self.sides, self.norms):
             if name.startswith(side + "."):
                 local = name[len(side) + 1:]
-                if local == self.norm_tensor:
+                if n is not None and local == self.norm_tensor:
                     # x / rms * w / sides: a division by a power of two is exact in every dtype here; otherwise the
                     # weight is kept in 32-bit
                     k = len(self.sides)
@@ -87,7 +90,7 @@ class SideBySide(Part):
     def finalize(self) -> None:
         for m in self.sides:
             m.finalize()
-        if len({n.weight.dtype for n in self.norms}) > 1:
+        if len({n.weight.dtype for n in self.norms if n is not None}) > 1:
             for n in self.norms:
                 n.weight = n.weight.float()
 

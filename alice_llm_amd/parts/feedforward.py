@@ -3,6 +3,9 @@
 (llama3.rs:6183-6186).  A second gated form, "swish_limited", bounds both branches first:
 g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1).  gate and up are stacked into one matrix at load so that one kernel reads
 the input once and applies the activation and the product in its epilogue.
+
+Dense MLP: down( act(up x) ), the activation as the epilogue of the first product; "relu_squared" is
+max(z, 0)^2.
 """
 from __future__ import annotations
 
@@ -72,3 +75,44 @@ class GatedMLP(Part):
                 and self.gate_up.can_write_fragments(x.shape[0]))
         h = self.gate_up(x, self.precision.act, out_fragments=frag)
         return self.down(h, torch.float32, allow_partials=True)
+
+
+# the activations of the ungated form are the matrix products' one-element epilogue; its parameter picks the function
+_UNARY_EPILOGUES = {"relu_squared": (ops.EPI_SOFTCAP, ops.UNARY_RELU2)}
+
+
+@FEED_FORWARDS.register("dense_mlp")
+class DenseMLP(Part):
+    graph_safe = True
+
+    def __init__(self, precision: Precision, *, hidden_size: int, intermediate_size: int, activation: str,
+                 tensor_names: Optional[Dict[str, str]] = None):
+        if activation not in _UNARY_EPILOGUES:
+            raise ValueError(f"dense_mlp has no kernel for activation '{activation}'; available: {sorted(_UNARY_EPILOGUES)}")
+        self.precision = precision
+        self.H, self.I = hidden_size, intermediate_size
+        self.names = dict({"up": "up_proj.weight", "down": "down_proj.weight"}, **(tensor_names or {}))
+        epi, param = _UNARY_EPILOGUES[activation]
+        self.up = Linear(hidden_size, intermediate_size, precision, epilogue=epi, epi_param=param)
+        self.down = Linear(intermediate_size, hidden_size, precision)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {self.names["up"]: ParamSpec((self.I, self.H)), self.names["down"]: ParamSpec((self.H, self.I))}
+
+    def assign(self, name: str, tensor: torch.Tensor) -> None:
+        if name == self.names["up"]:
+            self.up.load(tensor)
+        elif name == self.names["down"]:
+            self.down.load(tensor)
+        else:
+            raise KeyError(name)
+
+    def weight_bytes(self) -> int:
+        return self.up.nbytes() + self.down.nbytes()
+
+    @property
+    def accepts_fragment_activations(self) -> bool:
+        return self.up.accepts_fragment_input
+
+    def forward(self, x, ctx) -> torch.Tensor:
+        return self.down(self.up(x, self.precision.act), torch.float32, allow_partials=True)

@@ -78,6 +78,37 @@ class RotaryEncoding(Part):
         return True
 
 
+@POSITIONS.register("rope_pairs")
+class RotaryPairs(Part):
+    """Rotation in pairs of neighbouring dimensions (2i, 2i + 1), or of halves (i, i + R/2), over the first
+    `rotary_dim` dimensions of every q and k head: the pair (u, v) at position p becomes
+    (u cos a - v sin a, v cos a + u sin a), a = p * theta^(-2i / rotary_dim).  With `value_dim` the values are
+    turned too, over all their dimensions and with frequencies of their own, theta^(-2m / value_dim), by their
+    own position, and the attention kernel turns every head's output back by the query's position (so that a
+    value enters the output turned by the distance).  The tables are made on the host in 64-bit and kept in
+    32-bit; the attention mixer hands them to its kernels (`cos`, `sin`, `value_cos`, `value_sin`)."""
+    graph_safe = True
+
+    def __init__(self, precision: Precision, device, *, dim: int, theta: float, max_positions: int,
+                 rotary_dim: Optional[int] = None, value_dim: Optional[int] = None, interleaved: bool = True):
+        self.dim = dim
+        self.rotary_dim = dim if rotary_dim is None else int(rotary_dim)
+        if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= dim:
+            raise ValueError(f"rotated width {self.rotary_dim} must be even and at most {dim}")
+        if value_dim is not None and value_dim % 2:
+            raise ValueError(f"turned values need an even size, found {value_dim}")
+        self.theta, self.max_positions = float(theta), max_positions
+        self.value_dim, self.interleaved = value_dim, bool(interleaved)
+        self.cos, self.sin = self._tables(self.rotary_dim, device) if self.rotary_dim else (None, None)
+        self.value_cos, self.value_sin = self._tables(value_dim, device) if value_dim else (None, None)
+
+    def _tables(self, width: int, device):
+        i = torch.arange(width // 2, dtype=torch.float64)
+        ang = torch.arange(self.max_positions, dtype=torch.float64)[:, None] * (self.theta ** (-2.0 * i / width))[None, :]
+        return (torch.cos(ang).to(torch.float32).to(device).contiguous(),
+                torch.sin(ang).to(torch.float32).to(device).contiguous())
+
+
 @POSITIONS.register("none")
 class NoPositionEncoding(Part):
     graph_safe = True

@@ -70,6 +70,19 @@ def check_tensors(where: str, specs: Dict[str, ParamSpec], found: Dict[str, Tupl
     return unexpected
 
 
+def config_of_folder(folder: str):
+    """A model folder's configuration: config.json, and for an architecture some of whose sizes only the tensors
+    give (its configuration class has `with_tensor_shapes`), those sizes from the shapes in model.safetensors."""
+    config = load_config(folder)
+    if hasattr(config, "with_tensor_shapes"):
+        src = TensorSource(folder)
+        try:
+            config = config.with_tensor_shapes({k: tuple(src.info(k)[1]) for k in src.keys()})
+        finally:
+            src.close()
+    return config
+
+
 def _place(model, name: str, spec: ParamSpec, t: torch.Tensor) -> None:
     if spec.integer:
         t = t.to(torch.int32)
