@@ -7,13 +7,17 @@
 // alpha is exp(logsigmoid(z) / tau) with the full-precision functions, the state lives in float32 rows of the
 // cache, one per slot, and the norm is 32-bit.
 //
-// gla_kernel: a block of four waves per (sequence, head, 64 value columns) walks through the sequence's tokens
-// of the step with its part of the state in registers (thread (rg, lane) holds rows rg, rg + 4, ... of column
-// lane), reads the state once and writes it once; a single token is the same walk of one step.  The next
-// token's operands are fetched while the current one is worked on.  Which rows belong to the sequence and
-// which state row is its own are read on the device (cu_seqlens, slots), so a launch depends on sizes only.
-// With dv <= 64 the head's norm and gate are finished by the block itself; wider heads leave o in a float32
-// workspace for gla_finish_kernel (the norm needs every column of a head).
+// gla_kernel: a block of 256 threads per (sequence, head, CB value columns) walks through the sequence's tokens of
+// the step with its part of the state in registers: thread (rg, col) holds RPT neighbouring rows of one column,
+// reads them once and writes them once; a single token is the same walk of one step.  The tokens go through LDS
+// TC at a time: q, k and the decays of TC tokens are put there by all threads (the next TC tokens' operands are
+// already on their way from memory), every thread then updates its rows token by token, with no barrier between
+// the tokens, and keeps its TC partial read-outs, which meet in LDS once per TC tokens and are added up in the
+// order of the row groups.  CB is 64 where (sequences x heads) fill the chip, 16 otherwise (more blocks, fewer rows
+// a thread).  Which rows belong to the sequence and which state row is its own are read on the device
+// (cu_seqlens, slots), so a launch depends on sizes only.  With CB = 64 and dv <= 64 the head's norm and gate are
+// finished by the block itself; otherwise o is left in a float32 workspace for gla_finish_kernel (the norm needs
+// every column of a head).
 #include "common.h"
 #include "alice_hip.h"
 
@@ -22,16 +26,24 @@ namespace {
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 __device__ __forceinline__ float silu(float z) { return z / (1.f + expf(-z)); }
 
-template <int RPT, typename TW, typename TO>
+template <int CB, int RPT, int TC, typename TW, typename TO>
 __global__ __launch_bounds__(256) void gla_kernel(
     const float* __restrict__ rows, int row_w, int q_col, int k_col, int v_col, int g_col,
     const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale, float out_scale,
     const TW* __restrict__ norm_w, float eps, TO* __restrict__ out, float* __restrict__ o32,
     const int* __restrict__ cu_seqlens, const int* __restrict__ slots, float* __restrict__ S, int H, int d, int dv) {
-  __shared__ float sq[256], sk[256], sa[256];
-  __shared__ float red[4][64];
-  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, rg = tid >> 6;
-  const int j = blockIdx.z * 64 + lane;
+  constexpr int RG = 256 / CB;                 // row groups
+  constexpr int DP = RG * RPT;                 // rows the block covers (>= d)
+  constexpr int NL = TC * DP / 256;            // q / k / z elements a thread fetches per TC tokens
+  constexpr int NV = (TC * CB + 255) / 256;    // v elements, and read-outs, a thread handles per TC tokens
+  static_assert(RPT % 4 == 0 && (TC * DP) % 256 == 0, "rows are read four at a time");
+  __shared__ __align__(16) float sq[TC][DP];
+  __shared__ __align__(16) float sk[TC][DP];
+  __shared__ __align__(16) float sa[TC][DP];
+  __shared__ float sv[TC][CB];
+  __shared__ float red[TC][RG][CB];
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, col = tid % CB, rg = tid / CB;
+  const int j = blockIdx.z * CB + col;
   const bool col_ok = j < dv;
   const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
   if (t1 <= t0) return;
@@ -39,59 +51,97 @@ __global__ __launch_bounds__(256) void gla_kernel(
   float st[RPT];
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = rg + 4 * i;
+    const int r = rg * RPT + i;
     st[i] = (r < d && col_ok) ? Sh[(size_t)r * dv + j] : 0.f;
   }
-  const bool finish_here = gridDim.z == 1;
-  // this thread's operands of the token: element tid of q, k and z (tid < d), element j of v
-  float nq = 0.f, nk = 0.f, nz = 0.f, nv = 0.f;
-  auto fetch = [&](int t) {
-    const float* row = rows + (size_t)t * row_w;
-    if (tid < d) {
-      nq = row[q_col + h * d + tid];
-      nk = row[k_col + h * d + tid];
-      nz = z[(size_t)t * H * d + h * d + tid];
-    }
-    if (col_ok) nv = row[v_col + h * dv + j];
-  };
-  fetch(t0);
-  for (int t = t0; t < t1; ++t) {
-    if (tid < d) {
-      sq[tid] = nq * q_scale;
-      sk[tid] = nk;
-      sa[tid] = expf(log_sigmoid(nz + z_bias[h * d + tid]) * inv_tau);
-    }
-    const float vj = nv;
-    __syncthreads();
-    if (t + 1 < t1) fetch(t + 1);
-    float part = 0.f;
+  const bool finish_here = CB == 64 && gridDim.z == 1;
+  // what this thread fetches for TC tokens: element (t, r) = (idx / DP, idx % DP) of q, k and z; (t, c) of v
+  float pq[NL], pk[NL], pz[NL], pv[NV];
+  auto fetch = [&](int tc) {
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      const int r = rg + 4 * i;
-      if (r < d) {
-        st[i] = fmaf(sa[r], st[i], sk[r] * vj);
-        part = fmaf(st[i], sq[r], part);
+    for (int n = 0; n < NL; ++n) {
+      const int idx = tid + n * 256, t = tc + idx / DP, r = idx % DP;
+      pq[n] = pk[n] = pz[n] = 0.f;
+      if (t < t1 && r < d) {
+        const float* row = rows + (size_t)t * row_w;
+        pq[n] = row[q_col + h * d + r];
+        pk[n] = row[k_col + h * d + r];
+        pz[n] = z[(size_t)t * H * d + h * d + r];
       }
     }
-    red[rg][lane] = part;
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int idx = tid + n * 256, t = tc + idx / CB, c = blockIdx.z * CB + idx % CB;
+      pv[n] = (idx < TC * CB && t < t1 && c < dv) ? rows[(size_t)t * row_w + v_col + h * dv + c] : 0.f;
+    }
+  };
+  fetch(t0);
+  for (int tc = t0; tc < t1; tc += TC) {
+    const int n_tok = min(TC, t1 - tc);
+#pragma unroll
+    for (int n = 0; n < NL; ++n) {
+      const int idx = tid + n * 256, t = idx / DP, r = idx % DP;
+      sq[t][r] = pq[n] * q_scale;
+      sk[t][r] = pk[n];
+      // rows beyond d hold zeros and stay zero whatever their decay
+      sa[t][r] = r < d ? expf(log_sigmoid(pz[n] + z_bias[h * d + r]) * inv_tau) : 0.f;
+    }
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int idx = tid + n * 256;
+      if (idx < TC * CB) sv[idx / CB][idx % CB] = pv[n];
+    }
     __syncthreads();
-    if (rg == 0) {
-      const float o = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
-      if (finish_here) {
-        const float ss = wave_sum(col_ok ? o * o : 0.f);
-        if (col_ok) {
-          const float g = rows[(size_t)t * row_w + g_col + h * dv + j];
-          const float y = o / sqrtf(ss / (float)dv + eps) * load_f32(norm_w, j) * silu(g) * out_scale;
-          store_f32(out + (size_t)t * H * dv + h * dv, j, y);
+    if (tc + TC < t1) fetch(tc + TC);
+    float part[TC];
+#pragma unroll
+    for (int t = 0; t < TC; ++t) {
+      float p = 0.f;
+      if (t < n_tok) {
+        const float vj = sv[t][col];
+#pragma unroll
+        for (int i = 0; i < RPT; i += 4) {
+          const float4 a = *reinterpret_cast<const float4*>(&sa[t][rg * RPT + i]);
+          const float4 kk = *reinterpret_cast<const float4*>(&sk[t][rg * RPT + i]);
+          const float4 qq = *reinterpret_cast<const float4*>(&sq[t][rg * RPT + i]);
+          st[i] = fmaf(a.x, st[i], kk.x * vj);
+          p = fmaf(st[i], qq.x, p);
+          st[i + 1] = fmaf(a.y, st[i + 1], kk.y * vj);
+          p = fmaf(st[i + 1], qq.y, p);
+          st[i + 2] = fmaf(a.z, st[i + 2], kk.z * vj);
+          p = fmaf(st[i + 2], qq.z, p);
+          st[i + 3] = fmaf(a.w, st[i + 3], kk.w * vj);
+          p = fmaf(st[i + 3], qq.w, p);
         }
-      } else if (col_ok) {
-        o32[(size_t)t * H * dv + h * dv + j] = o;
+      }
+      part[t] = p;
+    }
+#pragma unroll
+    for (int t = 0; t < TC; ++t) red[t][rg][col] = part[t];
+    __syncthreads();
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int idx = tid + n * 256, t = idx / CB, c = idx % CB, jj = blockIdx.z * CB + c;
+      if (idx >= TC * CB) continue;            // (with CB = 64 a wave has one token: the branch is uniform)
+      float o = 0.f;
+#pragma unroll
+      for (int g = 0; g < RG; ++g) o += red[t][g][c];
+      const bool ok = t < n_tok && jj < dv;
+      const size_t at = (size_t)(tc + t) * H * dv + h * dv + jj;
+      if (finish_here) {
+        const float ss = wave_sum(ok ? o * o : 0.f);
+        if (ok) {
+          const float g = rows[(size_t)(tc + t) * row_w + g_col + h * dv + jj];
+          store_f32(out, at, o / sqrtf(ss / (float)dv + eps) * load_f32(norm_w, jj) * silu(g) * out_scale);
+        }
+      } else if (ok) {
+        o32[at] = o;
       }
     }
   }
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = rg + 4 * i;
+    const int r = rg * RPT + i;
     if (r < d && col_ok) Sh[(size_t)r * dv + j] = st[i];
   }
 }
@@ -116,9 +166,11 @@ __global__ __launch_bounds__(256) void gla_finish_kernel(const float* __restrict
 
 }  // namespace
 
+
 // rows: float32 [T, row_w] with q at q_col (H d), k at k_col (H d), v at v_col (H dv) and the gate at g_col (H dv);
 // z: float32 [T, H d], the decay's pre-activation without its bias z_bias [H d]; S: [n_slots, H, d, dv] float32;
-// out: [T, H dv] in out_dtype, times the constant out_scale; work: float32 [T, H dv], read only where dv > 64.
+// out: [T, H dv] in out_dtype, times the constant out_scale; work: float32 [T, H dv] (may be null where (sequences x
+// heads) fill the chip and dv <= 64: then nothing is read from it).
 extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, const float* z,
                          const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
                          int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
@@ -127,21 +179,30 @@ extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int
   ALICE_CHECK(rows && z && z_bias && norm_w && out && cu_seqlens && slots && S, "gla: a pointer is missing");
   ALICE_CHECK(T >= 0 && n_seqs >= 0 && n_slots >= 1 && H >= 1 && d >= 1 && dv >= 1, "gla: bad sizes");
   ALICE_CHECK(d <= 256, "gla: key size %d is beyond 256, the range of this kernel", d);
-  ALICE_CHECK(dv <= 64 || work != nullptr, "gla: value heads wider than 64 need the workspace");
   ALICE_CHECK(tau > 0.f, "gla: tau must be positive");
   ALICE_CHECK(min(min(q_col, k_col), min(v_col, g_col)) >= 0 && max(q_col, k_col) + H * d <= row_w && max(v_col, g_col) + H * dv <= row_w,
               "gla: rows of %d elements are too short for the heads", row_w);
-  ALICE_CHECK(H <= 65535 && ceil_div(dv, 64) <= 65535, "gla: too many heads for one launch");
+  ALICE_CHECK(H <= 65535 && dv <= 65535 * 16, "gla: too many heads for one launch");
   if (T == 0 || n_seqs == 0) return 0;
-  dim3 grid(n_seqs, H, ceil_div(dv, 64));
-#define GO(RPT, TW, TO)                                                                                                         \
-  gla_kernel<RPT, TW, TO><<<grid, 256, 0, stream>>>(rows, row_w, q_col, k_col, v_col, g_col, z, z_bias, 1.f / tau, q_scale, out_scale, \
-      (const TW*)norm_w, eps, (TO*)out, work, cu_seqlens, slots, S, H, d, dv)
-#define BY_D(TW, TO)                 \
-  do {                               \
-    if (d <= 64) GO(16, TW, TO);     \
-    else if (d <= 128) GO(32, TW, TO); \
-    else GO(64, TW, TO);             \
+  // 64 columns a block where that fills the chip, else 16 (four times the blocks)
+  const bool wide = (long)n_seqs * H * ceil_div(dv, 64) >= 512;
+  const bool finish_here = wide && dv <= 64;
+  ALICE_CHECK(finish_here || work != nullptr, "gla: this shape needs the workspace");
+  dim3 grid(n_seqs, H, ceil_div(dv, wide ? 64 : 16));
+#define GO(CB, RPT, TC, TW, TO)                                                                                                  \
+  gla_kernel<CB, RPT, TC, TW, TO><<<grid, 256, 0, stream>>>(rows, row_w, q_col, k_col, v_col, g_col, z, z_bias, 1.f / tau, q_scale, \
+      out_scale, (const TW*)norm_w, eps, (TO*)out, work, cu_seqlens, slots, S, H, d, dv)
+#define BY_D(TW, TO)                              \
+  do {                                            \
+    if (wide) {                                   \
+      if (d <= 64) GO(64, 16, 8, TW, TO);         \
+      else if (d <= 128) GO(64, 32, 4, TW, TO);   \
+      else GO(64, 64, 4, TW, TO);                 \
+    } else {                                      \
+      if (d <= 64) GO(16, 4, 16, TW, TO);         \
+      else if (d <= 128) GO(16, 8, 16, TW, TO);   \
+      else GO(16, 16, 8, TW, TO);                 \
+    }                                             \
   } while (0)
   if (w_dtype == DT_F32 && out_dtype == DT_F32) BY_D(float, float);
   else if (w_dtype == DT_F32) BY_D(float, bf16_t);
@@ -150,9 +211,9 @@ extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int
 #undef BY_D
 #undef GO
   ALICE_LAUNCH_CHECK();
-  if (dv > 64) {
+  if (!finish_here) {
     dim3 g2(T, H);
-#define FIN(TW, TO) gla_finish_kernel<TW, TO><<<g2, 256, 0, stream>>>(work, rows, row_w, g_col, (const TW*)norm_w, eps, out_scale, (TO*)out, H, dv)
+#define FIN(TW, TO) gla_finish_kernel<TW, TO><<<g2, dv > 128 ? 256 : 64, 0, stream>>>(work, rows, row_w, g_col, (const TW*)norm_w, eps, out_scale, (TO*)out, H, dv)
     if (w_dtype == DT_F32 && out_dtype == DT_F32) FIN(float, float);
     else if (w_dtype == DT_F32) FIN(float, bf16_t);
     else if (out_dtype == DT_F32) FIN(bf16_t, float);

@@ -633,7 +633,7 @@ def gla(rows: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, norm_w: torch
         raise HipLibraryError("cu_seqlens and slots are too short for the step's sequences")
     n_slots = S.shape[0]
     _dev(S, "S", torch.float32, (n_slots, H, d, dv))
-    work = torch.empty((T, H * dv), dtype=torch.float32, device=rows.device) if dv > 64 else None
+    work = torch.empty((T, H * dv), dtype=torch.float32, device=rows.device)
     q_col, k_col, v_col, g_col = (int(c) for c in columns)
     _call("alice_gla", rows.data_ptr(), rows.shape[1], q_col, k_col, v_col, g_col, z.data_ptr(), z_bias.data_ptr(), float(tau),
           float(q_scale), float(out_scale), norm_w.data_ptr(), dtype_code(norm_w.dtype), float(eps), out.data_ptr(), dtype_code(out.dtype),

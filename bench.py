@@ -11,6 +11,8 @@ device-to-device copy and a large bfloat16 matrix product of the vendor library)
 of the other configurations: the 2B shape at contexts from 8,000, 16 unequal prompts at the 9B shape, and 8 prompts
 of 6,000 tokens, past the window, at the 27B shape.
 
+    python bench.py --telulorn w2048,w4096
+        instead of the above: the Telulorn design beside Novotar and Gemma 2 at equal layer sizes, in a line of its own
     python bench.py --novotar w2048,w4096
         instead of the above: prefill and decode throughput of the Novotar design at layer sizes of real models
         (random weights, a few layers), beside Gemma 2 at equal sizes; prints a line of its own
@@ -310,13 +312,33 @@ def novotar_pair_configs(size, vocab=32768, window=1024):
     return nov, gem
 
 
-def novotar_bench(sizes, dtype, steps, warmup):
+def telulorn_configs(size, vocab=32768, window=1024):
+    """A Telulorn configuration of four layers (side-by-side mixer, attention, side-by-side mixer, attention), the middle
+    two run twice (six layer runs), at the sizes of novotar_pair_configs: the same width, feed-forward, attention
+    heads and window (as the chunk of the one mixer and the window of the other, which keeps 64 first positions);
+    the recurrence with the matrix memory's heads and head sizes."""
+    z = NOVOTAR_SIZES[size]
+    heads = {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5}
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    par = {"type": "parallel", "mlp": mlp,
+           "mixer": {"left": dict(heads, mask={"size": window}), "left_scale": 1.2, "right_scale": 1.1,
+                     "right": {"heads": z["mheads"], "dim": z["mdim"], "vdim": z["mvdim"], "tau": 16.0, "rank": 64}}}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": dict(heads, mask={"size": window, "keep_first": 64}, rot={"base": 10000.0, "dims": z["dim"] // 2})}
+    return {"architecture": "Telulorn", "vocab": vocab, "width": z["width"], "norm": {"eps": 1e-6},
+            "layers": [par, att, par, att], "loop": {"start": 1, "stop": 3, "times": 2}}
+
+
+def novotar_bench(sizes, dtype, steps, warmup, with_telulorn=False):
     out = {}
     for size in sizes:
         if size not in NOVOTAR_SIZES:
-            raise SystemExit(f"--novotar: unknown size '{size}'; known: {sorted(NOVOTAR_SIZES)}")
+            raise SystemExit(f"unknown size '{size}'; known: {sorted(NOVOTAR_SIZES)}")
         res = {}
-        for name, raw in zip(("novotar", "gemma2"), novotar_pair_configs(size)):
+        models = list(zip(("novotar", "gemma2"), novotar_pair_configs(size)))
+        if with_telulorn:
+            models.insert(0, ("telulorn", telulorn_configs(size)))
+        for name, raw in models:
             run = Run(None, None, dtype, raw=raw)
             r = {"weights_gb": round(run.weight_bytes / 1e9, 3), "layer_runs": len(run.model.lm.plan.schedule)}
             for T in (2048, 8192):
@@ -389,6 +411,8 @@ def main() -> int:
                     help="shorter runs of other configurations, reported under 'shapes' ('' for none)")
     ap.add_argument("--novotar", default="", help="sizes (w2048,w4096): measure the Novotar design beside Gemma 2 at equal "
                     "sizes instead of the default workload, and print a line of its own")
+    ap.add_argument("--telulorn", default="", help="sizes (w2048,w4096): measure the Telulorn design beside Novotar and Gemma 2 at "
+                    "equal sizes instead of the default workload, and print a line of its own")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own copy and matrix-product rates")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -397,6 +421,13 @@ def main() -> int:
 
     import torch
     torch.cuda.set_device(0)
+    if args.telulorn:
+        steps = min(args.steps, 64)
+        res = novotar_bench([x for x in args.telulorn.split(",") if x], args.dtype, steps, min(args.warmup, 5), with_telulorn=True)
+        print(json.dumps({"metric": "Telulorn beside Novotar and Gemma 2 at equal layer sizes: prefill and decode, random weights",
+                          "unit": "tokens/s", "n_gpus": 1, "steps": steps, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                          "data": "synthetic (uniform random token ids, random weights)", "sizes": res}), flush=True)
+        return 0
     if args.novotar:
         steps = min(args.steps, 64)
         res = novotar_bench([x for x in args.novotar.split(",") if x], args.dtype, steps, min(args.warmup, 5))

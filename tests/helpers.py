@@ -235,3 +235,129 @@ def novotar_pair(name: str, dtype: str, seed: int = 0, device="cuda"):
     plain = PlainNovotar(raw, {k: v.double() for k, v in tensors.items()})
     model = model_from_tensors(cfg, {k: v.to(device) for k, v in tensors.items()}, dtype)
     return model, plain
+
+
+# --------------------------------------------------------------------------- Telulorn test configurations
+# A: a loop in the middle run twice; grouped kv heads; value heads twice / half the key size; a chunk and a window
+#    shorter than a page; a part of the head rotated; one layer without a feed-forward; side factors other than 1.
+# B: no loop; kv heads = heads; sizes that fit no tile (width 72, heads of 20 / 28 / 12); the whole head rotated; a
+#    window and a chunk longer than a page; tau 1; both side factors 1.
+# C: sizes that suit the matrix cores; a loop over every layer run three times; one kv head; a chunk of exactly a
+#    page; kept first positions that reach into the second page; value heads of the recurrence wider than 64.
+# D: an attention layer first; a loop over the first layer alone; a layer without any mask and one whose window
+#    keeps no first positions; keys of the recurrence wider than 128; three query heads a kv head.
+def _tl_par(left, right, mlp, ls=1.0, rs=1.0):
+    return {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": ls, "right_scale": rs}, "mlp": mlp}
+
+
+def _tl_a():
+    le = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.3, "mask": {"size": 7}}
+    ri = {"heads": 2, "dim": 16, "vdim": 32, "tau": 4.0, "rank": 8}
+    at = {"heads": 4, "kv_heads": 1, "dim": 32, "vdim": 16, "scale": 0.2, "mask": {"size": 9, "keep_first": 3},
+          "rot": {"base": 100.0, "dims": 16}}
+    mlp = {"kind": "dense", "ff": 96}
+    return {"architecture": "Telulorn", "vocab": 97, "width": 64, "norm": {"eps": 1e-6},
+            "layers": [_tl_par(le, ri, mlp, 0.8, 1.3), {"type": "attention", "mixer": at, "mlp": mlp}, _tl_par(le, ri, None, 1.5, 0.7)],
+            "loop": {"start": 1, "stop": 3, "times": 2}}
+
+
+def _tl_b():
+    le = {"heads": 3, "kv_heads": 3, "dim": 20, "vdim": 28, "scale": 0.25, "mask": {"size": 100}}
+    ri = {"heads": 3, "dim": 12, "vdim": 20, "tau": 1.0, "rank": 5}
+    at = {"heads": 3, "kv_heads": 3, "dim": 20, "vdim": 20, "scale": 0.3, "mask": {"size": 70, "keep_first": 5},
+          "rot": {"base": 10000.0, "dims": 20}}
+    mlp = {"kind": "dense", "ff": 100}
+    return {"architecture": "Telulorn", "vocab": 130, "width": 72, "norm": {"eps": 1e-5},
+            "layers": [_tl_par(le, ri, mlp), {"type": "attention", "mixer": at, "mlp": mlp}]}
+
+
+def _tl_c():
+    le = {"heads": 4, "kv_heads": 1, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 64}}
+    ri = {"heads": 2, "dim": 64, "vdim": 128, "tau": 16.0, "rank": 32}
+    at = {"heads": 4, "kv_heads": 1, "dim": 64, "vdim": 128, "scale": 0.125, "mask": {"size": 40, "keep_first": 70},
+          "rot": {"base": 500.0, "dims": 32}}
+    mlp = {"kind": "dense", "ff": 256}
+    return {"architecture": "Telulorn", "vocab": 300, "width": 128, "norm": {"eps": 1e-6},
+            "layers": [{"type": "attention", "mixer": at, "mlp": mlp}, _tl_par(le, ri, mlp, 1.1, 0.9)],
+            "loop": {"start": 0, "stop": 2, "times": 3}}
+
+
+def _tl_d():
+    le = {"heads": 3, "kv_heads": 1, "dim": 24, "vdim": 24, "scale": 0.2}
+    ri = {"heads": 1, "dim": 136, "vdim": 24, "tau": 8.0, "rank": 3}
+    at = {"heads": 6, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.25, "mask": {"size": 33}, "rot": {"base": 50.0, "dims": 8}}
+    free = {k: v for k, v in at.items() if k != "mask"}
+    mlp = {"kind": "dense", "ff": 80}
+    return {"architecture": "Telulorn", "vocab": 61, "width": 48, "norm": {"eps": 1e-6},
+            "layers": [{"type": "attention", "mixer": at, "mlp": mlp}, _tl_par(le, ri, mlp, 1.2, 1.0),
+                       {"type": "attention", "mixer": free, "mlp": None}],
+            "loop": {"start": 0, "stop": 1, "times": 2}}
+
+
+TELULORN = {"tl-a": _tl_a, "tl-b": _tl_b, "tl-c": _tl_c, "tl-d": _tl_d}
+
+
+def telulorn_tensors(raw: dict, seed: int):
+    """Random tensors for a Telulorn configuration, by name, in bfloat16 on the CPU: matrices N(0, gain^2 / inputs)
+    with gains that make every mechanism matter (sharp softmaxes, gates that open and close, sinks of the scores'
+    order, a head mix far from the identity, decays from fast to almost none), norm weights around 1."""
+    import alice_llm_amd as alice
+    from alice_llm_amd.engine.model import CausalLM
+    from alice_llm_amd.parts import Precision
+    cfg = alice.config_from_dict(raw)
+    specs = CausalLM(cfg.plan(), Precision.of("float32"), "cpu").param_specs()
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, spec in specs.items():
+        shape = tuple(spec.shape)
+        r = torch.randn(shape, generator=g)
+        if name.endswith(".sink"):
+            t = 1.5 * r
+        elif name.endswith("a2.b"):
+            t = 2.0 + 3.0 * r                       # sigmoid(.)^(1/tau) from about 0.5 to almost 1
+        elif name.endswith(".talk"):
+            t = torch.eye(shape[0]) * 0.7 + 0.4 * r
+        elif name == "loop.step":
+            t = 0.3 * r
+        elif len(shape) == 1:
+            t = 0.5 * r if name.endswith(".b") else 1.0 + 0.2 * r
+        elif name == "embed":
+            t = r * 0.5
+        else:
+            gain = 2.5 if name.endswith((".q", ".k", ".g", ".a2")) else 1.0
+            t = r * gain / shape[1] ** 0.5
+        out[name] = t.to(torch.bfloat16)
+    return cfg, out
+
+
+def telulorn_pair(name: str, dtype: str, seed: int = 0, device="cuda"):
+    """(the package's model, the plain model) on the same tensors."""
+    from plain.telulorn_plain import PlainTelulorn
+    raw = TELULORN[name]()
+    cfg, tensors = telulorn_tensors(raw, seed)
+    plain = PlainTelulorn(raw, tensors)
+    model = model_from_tensors(cfg, {k: v.to(device) for k, v in tensors.items()}, dtype)
+    return model, plain
+
+
+def telulorn_folder(name: str, seed: int = 0) -> str:
+    """A model folder (config.json without the decay projection's middle width, which the tensors give;
+    model.safetensors in bfloat16) of a Telulorn test configuration."""
+    global _TMP
+    key = ("telulorn", name, seed)
+    if key not in _FOLDERS:
+        from safetensors.torch import save_file
+        if _TMP is None:
+            _TMP = tempfile.TemporaryDirectory(prefix="alice_tests_")
+        folder = os.path.join(_TMP.name, f"{name}-{seed}")
+        os.makedirs(folder, exist_ok=True)
+        raw = TELULORN[name]()
+        _, tensors = telulorn_tensors(raw, seed)
+        for l in raw["layers"]:
+            if l["type"] == "parallel":
+                l["mixer"]["right"].pop("rank", None)
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(raw, f)
+        save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
+        _FOLDERS[key] = folder
+    return _FOLDERS[key]

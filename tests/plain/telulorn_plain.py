@@ -284,3 +284,26 @@ def read_model(folder: str):
     with open(os.path.join(folder, "config.json")) as f:
         config = json.load(f)
     return config, read_safetensors(os.path.join(folder, "model.safetensors"))
+
+
+class PlainTelulorn:
+    """The plain model on given tensors (64-bit)."""
+
+    def __init__(self, config: dict, tensors: dict):
+        self.c = config
+        self.w = {k: (v.to(DT) if v.is_floating_point() else v) for k, v in tensors.items()}
+
+    @classmethod
+    def from_folder(cls, folder: str) -> "PlainTelulorn":
+        return cls(*read_model(folder))
+
+    def forward(self, tokens, return_layers: bool = False):
+        return forward(self.c, self.w, tokens, return_layers)
+
+    def greedy(self, prompt, n: int):
+        seq, out = list(prompt), []
+        for _ in range(n):
+            tok = int(self.forward(seq)[-1].argmax())
+            out.append(tok)
+            seq.append(tok)
+        return out
