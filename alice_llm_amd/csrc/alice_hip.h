@@ -125,6 +125,15 @@ int alice_attention_masked(const void* q, int dtype, const void* k_pool, const v
                            int dv, const float* gate, int gate_stride, int gate_mode, float out_scale, int chunk,
                            int keep_first, const float* sink, const float* vrot_cos, const float* vrot_sin,
                            float* out32, hipStream_t stream);
+// alice_attention_masked's result for bfloat16 prompts on the matrix cores (attention_tiled.hip): the step's tokens are
+// those of n_seqs sequences in order (cu_seqlens), each at consecutive positions; head sizes multiples of 8 up to 256.
+int alice_attention_tiled_supported(int d, int dv);
+int alice_attention_tiled(const void* q, const void* k_pool, const void* v_pool, void* out, float* out32,
+                          const int* positions, const int* cu_seqlens, const int* block_table, int bt_stride,
+                          int T, int n_seqs, int nH, int nKV, int d, int dv, int page_size, float scale, int window,
+                          int chunk, int keep_first, const float* bias_slopes, const float* sink,
+                          const float* vrot_cos, const float* vrot_sin, const float* gate, int gate_stride,
+                          int gate_mode, float out_scale, hipStream_t stream);
 // out[t, h, e] = out_scale * sigmoid(gate[t, h dv + e]) * sum_g talk[h, g] a[t, g, kv head of h, e] (gate optional)
 int alice_mix_heads(const float* a, const float* talk, const float* gate, int gate_stride, float out_scale, void* out,
                     int dtype, int T, int nH, int nKV, int dv, int full_precision, hipStream_t stream);

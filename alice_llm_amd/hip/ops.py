@@ -58,6 +58,8 @@ def _declare(lib) -> None:
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, P],
         "alice_head_gate": [P, I, P, I, I, I, I, P],
         "alice_attention_masked": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, I, F, I, I, P, P, P, P, P],
+        "alice_attention_tiled": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, I, P, P, P, P, P, I, I, F, P],
+        "alice_attention_tiled_supported": [I, I],
         "alice_mix_heads": [P, P, P, I, F, P, I, I, I, I, I, I, P],
         "alice_qkv_prepare": [P, I, I, P, P, P, P, I, P, P, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "alice_add_rows": [P, P, P, I, I, P],
@@ -529,6 +531,68 @@ def attention_masked(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
           2 if gate_per_element else 1, float(out_scale), int(chunk or 0), int(keep_first or 0), None if sink is None else sink.data_ptr(),
           None if value_cos is None else value_cos.data_ptr(), None if value_sin is None else value_sin.data_ptr(),
           None if per_value_head is None else per_value_head.data_ptr(), _stream())
+
+
+def attention_tiled_supported(dtype: torch.dtype, head_dim: int, value_head_dim: int) -> bool:
+    """Whether attention_tiled takes these operands: bfloat16 and head sizes that are multiples of 8 up to 256."""
+    return dtype == torch.bfloat16 and bool(library().alice_attention_tiled_supported(int(head_dim), int(value_head_dim)))
+
+
+def attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: Optional[torch.Tensor], ctx,
+                    block_table: torch.Tensor, *, num_heads: int, scale: float, window: Optional[int] = None,
+                    chunk: Optional[int] = None, keep_first: int = 0, bias_slopes: Optional[torch.Tensor] = None,
+                    sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, gate_per_element: bool = False,
+                    out_scale: float = 1.0, value_cos: Optional[torch.Tensor] = None, value_sin: Optional[torch.Tensor] = None,
+                    per_value_head: Optional[torch.Tensor] = None) -> None:
+    """attention_masked's result for bfloat16 prompts by the matrix-core kernel over the row-major cache (see
+    attention_tiled.hip): `ctx` gives positions, cu_seqlens and the step's sizes; every sequence's tokens stand at
+    consecutive positions.  The other arguments are attention_masked's."""
+    T = q.shape[0]
+    if k_pool.dim() != 4 or v_pool.dim() != 4:
+        raise HipLibraryError("k_pool must be [pages, nKV, page, d]")
+    n_pages, nKV, page_size, d = k_pool.shape
+    dv = v_pool.shape[3]
+    _dev(q, "q", torch.bfloat16, (T, num_heads * d))
+    _dev(k_pool, "k_pool", torch.bfloat16)
+    _dev(v_pool, "v_pool", torch.bfloat16, tuple(k_pool.shape[:3]) + (dv,))
+    if per_value_head is not None:
+        _dev(per_value_head, "per_value_head", torch.float32, (T, num_heads, nKV, dv))
+        if gate is not None:
+            raise HipLibraryError("per-value-head outputs take no gate: the mix that follows does")
+    else:
+        _dev(out, "out", torch.bfloat16, (T, num_heads * dv))
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        need = num_heads * dv if gate_per_element else num_heads
+        if (not gate.is_cuda or gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < need
+                or gate.stride(1) != 1 or gate.stride(0) < need):
+            raise HipLibraryError(f"gate must be [{T}, >= {need}] float32 with unit column stride")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
+    _dev(ctx.positions, "positions", torch.int32)
+    _dev(ctx.cu_seqlens, "cu_seqlens", torch.int32)
+    _dev(block_table, "block_table", torch.int32)
+    if ctx.positions.numel() < T or ctx.cu_seqlens.numel() < ctx.n_seqs + 1:
+        raise HipLibraryError("positions and cu_seqlens are too short for the step")
+    if block_table.dim() != 2 or block_table.shape[0] < ctx.n_seqs or ctx.max_position // page_size >= block_table.shape[1]:
+        raise HipLibraryError(f"position {ctx.max_position} is beyond the block table {tuple(block_table.shape)}")
+    if bias_slopes is not None:
+        _dev(bias_slopes, "bias_slopes", torch.float32, (num_heads,))
+    if sink is not None:
+        _dev(sink, "sink", torch.float32, (num_heads,))
+    if value_cos is not None:
+        if dv % 2 or value_cos.dim() != 2 or value_cos.shape[1] != dv // 2 or value_sin.shape != value_cos.shape:
+            raise HipLibraryError(f"value tables must be [positions, {dv // 2}]")
+        _dev(value_cos, "value_cos", torch.float32)
+        _dev(value_sin, "value_sin", torch.float32)
+        if ctx.max_position >= value_cos.shape[0]:
+            raise HipLibraryError(f"position {ctx.max_position} is beyond the rotation tables ({value_cos.shape[0]} positions)")
+    _call("alice_attention_tiled", q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), None if out is None else out.data_ptr(),
+          None if per_value_head is None else per_value_head.data_ptr(), ctx.positions.data_ptr(), ctx.cu_seqlens.data_ptr(),
+          block_table.data_ptr(), block_table.shape[1], T, int(ctx.n_seqs), num_heads, nKV, d, dv, page_size, float(scale),
+          int(window or 0), int(chunk or 0), int(keep_first or 0), None if bias_slopes is None else bias_slopes.data_ptr(),
+          None if sink is None else sink.data_ptr(), None if value_cos is None else value_cos.data_ptr(),
+          None if value_sin is None else value_sin.data_ptr(), gate_ptr, int(gate_stride), 2 if gate_per_element else 1,
+          float(out_scale), _stream())
 
 
 def mix_heads(a: torch.Tensor, talk: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, *,

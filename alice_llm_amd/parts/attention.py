@@ -235,19 +235,28 @@ class Attention(Part):
             g0 = self.q_dim + self.kv_dim + self.v_dim
             gate = rows[:, g0:g0 + self.n_gate]
         out = torch.empty((T, self.o_in), dtype=act, device=dev)
-        common = dict(num_heads=self.nH, scale=self.scale, softcap=self.softcap, window=self.window, chunk=self.chunk,
-                      keep_first=self.keep_first, max_position=ctx.max_position, full_precision=self.precision.full,
+        common = dict(num_heads=self.nH, scale=self.scale, window=self.window, chunk=self.chunk, keep_first=self.keep_first,
                       bias_slopes=self._slopes, sink=self.sink, value_cos=getattr(pos, "value_cos", None),
                       value_sin=getattr(pos, "value_sin", None))
+        # steps with pieces of several tokens: the matrix-core kernel (bfloat16); steps of single tokens and the 32-bit
+        # path: the 32-bit kernel (the choice must not depend on the sizes that a captured step rounds up)
+        tiled = (not ctx.is_decode and self.softcap is None and not self.precision.full
+                 and ops.attention_tiled_supported(act, self.d, self.dv))
+
+        def attend(out_, per_, **more):
+            if tiled:
+                ops.attention_tiled(q, cache.k, cache.v, out_, ctx, cache.block_table, per_value_head=per_, **common, **more)
+            else:
+                ops.attention_masked(q, cache.k, cache.v, out_, ctx.positions, ctx.seq_of_token, cache.block_table,
+                                     per_value_head=per_, softcap=self.softcap, max_position=ctx.max_position,
+                                     full_precision=self.precision.full, **common, **more)
         if self.has_talk:
             # every head's weights on each kv head's values, then the mix of the heads with the gate behind it
-            per = torch.empty((T, self.nH, self.nKV, self.dv), dtype=torch.float32, device=dev)
-            ops.attention_masked(q, cache.k, cache.v, None, ctx.positions, ctx.seq_of_token, cache.block_table,
-                                 per_value_head=per, **common)
             if self.output_gate == "head":
                 raise NotImplementedError("attention: mixed heads take an elementwise gate or none")
+            per = torch.empty((T, self.nH, self.nKV, self.dv), dtype=torch.float32, device=dev)
+            attend(None, per)
             ops.mix_heads(per, self.talk, gate, out, full_precision=self.precision.full, out_scale=self.output_scale)
         else:
-            ops.attention_masked(q, cache.k, cache.v, out, ctx.positions, ctx.seq_of_token, cache.block_table, gate=gate,
-                                 gate_per_element=self.output_gate == "elementwise", out_scale=self.output_scale, **common)
+            attend(out, None, gate=gate, gate_per_element=self.output_gate == "elementwise", out_scale=self.output_scale)
         return self.o(out, torch.float32, allow_partials=True)

@@ -83,6 +83,24 @@ def _paged(k, v, page, scatter_seed):
     return kp.to(DEV), vp.to(DEV), order.to(torch.int32)[None].to(DEV)
 
 
+class _Pieces:
+    """What the matrix-core prompt kernel reads of a step: pieces of one sequence as if they were sequences of a step."""
+
+    def __init__(self, pieces, T):
+        cu = [0]
+        for a, b in pieces:
+            cu.append(cu[-1] + b - a)
+        self.positions = torch.cat([torch.arange(a, b) for a, b in pieces]).to(torch.int32).to(DEV)
+        self.cu_seqlens = torch.tensor(cu, dtype=torch.int32, device=DEV)
+        self.n_seqs, self.max_position, self.rows = len(pieces), T - 1, torch.cat([torch.arange(a, b) for a, b in pieces])
+
+
+def _pieces_of(T, edges):
+    """The whole prompt as one piece; then pieces that start and end around every edge, as sequences of one step."""
+    cuts = sorted({0, T} | {p for e in edges for p in (e - 1, e, e + 2) if 0 < p < T})
+    return [[(0, T)], list(zip(cuts[:-1], cuts[1:]))]
+
+
 def _rows_of(T, edges):
     """A whole prompt, its last token alone, and the single tokens around every edge."""
     out = [slice(0, T), slice(T - 1, T)]
@@ -132,6 +150,17 @@ def test_window_with_kept_first_positions_sink_and_turned_values(dtype, window, 
                              value_cos=vc, value_sin=vs)
         err = max_err(out.view(n, H, dv), ref[rows])
         assert err < (3e-5 if dtype == "float32" else 8e-2), (rows, err)
+    if dtype == "bfloat16":                     # the matrix-core kernel of prompts: whole, and in pieces around the edges
+        for pieces in _pieces_of(T, [mark + window, keep + window, 64]):
+            ctx = _Pieces(pieces, T)
+            n = ctx.rows.numel()
+            out = torch.empty(n, H * dv, dtype=dt, device=DEV)
+            ops.attention_tiled(q[ctx.rows].reshape(n, H * d).contiguous().to(DEV), kp, vp, out, ctx, bt.expand(ctx.n_seqs, -1).contiguous(),
+                                num_heads=H, scale=0.5, window=window, keep_first=keep, sink=sink.to(DEV),
+                                gate=gate.to(DEV)[ctx.rows][:, :H * dv], gate_per_element=True, out_scale=1.25,
+                                value_cos=vc, value_sin=vs)
+            err = max_err(out.view(n, H, dv), ref[ctx.rows])
+            assert err < 8e-2, (len(pieces), err)
     if mark + window < T:
         assert (ref[mark + window - 1] - ref[mark + window]).abs().max() > 0.3          # the markers do show
     if keep and keep + window < T:
@@ -175,6 +204,17 @@ def test_chunks_distance_term_and_mixed_heads(dtype, chunk, T):
         ops.mix_heads(per, talk.to(DEV), gate.to(DEV)[rows].contiguous(), out, full_precision=dtype == "float32", out_scale=0.75)
         err = max_err(out.view(n, H, dv), ref[rows])
         assert err < (3e-5 if dtype == "float32" else 8e-2), (rows, err)
+    if dtype == "bfloat16":
+        for pieces in _pieces_of(T, [last + 1, first, 64]):
+            ctx = _Pieces(pieces, T)
+            n = ctx.rows.numel()
+            per = torch.empty(n, H, G, dv, dtype=torch.float32, device=DEV)
+            out = torch.empty(n, H * dv, dtype=dt, device=DEV)
+            ops.attention_tiled(q[ctx.rows].reshape(n, H * d).contiguous().to(DEV), kp, vp, None, ctx, bt.expand(ctx.n_seqs, -1).contiguous(),
+                                num_heads=H, scale=0.5, chunk=chunk, bias_slopes=slopes.float().to(DEV), per_value_head=per)
+            ops.mix_heads(per, talk.to(DEV), gate.to(DEV)[ctx.rows].contiguous(), out, full_precision=False, out_scale=0.75)
+            err = max_err(out.view(n, H, dv), ref[ctx.rows])
+            assert err < 8e-2, (len(pieces), err)
     if last + 1 < T:
         assert (ref[last] - ref[last + 1]).abs().max() > 0.3
 
