@@ -134,6 +134,18 @@ int alice_attention_tiled(const void* q, const void* k_pool, const void* v_pool,
                           int chunk, int keep_first, const float* bias_slopes, const float* sink,
                           const float* vrot_cos, const float* vrot_sin, const float* gate, int gate_stride,
                           int gate_mode, float out_scale, hipStream_t stream);
+// alice_attention_masked's result for single tokens with the keys split over blocks (attention_split.hip), either
+// dtype, 32-bit arithmetic; max_keys: the most keys any token of the step sees; work: alice_attention_split_workspace
+// floats (runs = alice_attention_split_runs(max_keys)).
+int alice_attention_split_supported(int dtype, int nH, int nKV, int d, int dv);
+int alice_attention_split_runs(int max_keys);
+long alice_attention_split_workspace(int T, int nH, int nKV, int dv, int runs, int per_value_head);
+int alice_attention_split(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out, float* out32,
+                          const int* positions, const int* seq_of_token, const int* block_table, int bt_stride,
+                          int T, int nH, int nKV, int d, int dv, int page_size, float scale, int window, int chunk,
+                          int keep_first, int max_keys, const float* bias_slopes, const float* sink,
+                          const float* vrot_cos, const float* vrot_sin, const float* gate, int gate_stride,
+                          int gate_mode, float out_scale, float* work, hipStream_t stream);
 // out[t, h, e] = out_scale * sigmoid(gate[t, h dv + e]) * sum_g talk[h, g] a[t, g, kv head of h, e] (gate optional)
 int alice_mix_heads(const float* a, const float* talk, const float* gate, int gate_stride, float out_scale, void* out,
                     int dtype, int T, int nH, int nKV, int dv, int full_precision, hipStream_t stream);

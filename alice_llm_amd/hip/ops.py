@@ -60,6 +60,9 @@ def _declare(lib) -> None:
         "alice_attention_masked": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, I, F, I, I, P, P, P, P, P],
         "alice_attention_tiled": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, I, P, P, P, P, P, I, I, F, P],
         "alice_attention_tiled_supported": [I, I],
+        "alice_attention_split": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, I, P, P, P, P, P, I, I, F, P, P],
+        "alice_attention_split_supported": [I, I, I, I, I],
+        "alice_attention_split_runs": [I],
         "alice_mix_heads": [P, P, P, I, F, P, I, I, I, I, I, I, P],
         "alice_qkv_prepare": [P, I, I, P, P, P, P, I, P, P, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "alice_add_rows": [P, P, P, I, I, P],
@@ -77,6 +80,8 @@ def _declare(lib) -> None:
         fn.restype = I
     lib.alice_attention_decode_workspace.argtypes = [I, I, I, I]
     lib.alice_attention_decode_workspace.restype = L
+    lib.alice_attention_split_workspace.argtypes = [I, I, I, I, I, I]
+    lib.alice_attention_split_workspace.restype = L
     lib.alice_mlstm_chunks_workspace.argtypes = [I, I, I, I, I, I]
     lib.alice_mlstm_chunks_workspace.restype = L
 
@@ -593,6 +598,76 @@ def attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
           None if sink is None else sink.data_ptr(), None if value_cos is None else value_cos.data_ptr(),
           None if value_sin is None else value_sin.data_ptr(), gate_ptr, int(gate_stride), 2 if gate_per_element else 1,
           float(out_scale), _stream())
+
+
+def attention_split_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int, value_head_dim: int) -> bool:
+    """Whether attention_split takes these operands: groups of at most 16 query heads a kv head, head sizes that are
+    multiples of 16 bytes up to 256."""
+    return bool(library().alice_attention_split_supported(dtype_code(dtype), int(num_heads), int(num_kv_heads), int(head_dim),
+                                                          int(value_head_dim)))
+
+
+def attention_split(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, out: Optional[torch.Tensor],
+                    positions: torch.Tensor, seq_of_token: torch.Tensor, block_table: torch.Tensor, *, num_heads: int,
+                    scale: float, max_position: int, max_keys: int, window: Optional[int] = None, chunk: Optional[int] = None,
+                    keep_first: int = 0, bias_slopes: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+                    gate: Optional[torch.Tensor] = None, gate_per_element: bool = False, out_scale: float = 1.0,
+                    value_cos: Optional[torch.Tensor] = None, value_sin: Optional[torch.Tensor] = None,
+                    per_value_head: Optional[torch.Tensor] = None) -> None:
+    """attention_masked's result with the keys split over blocks (see attention_split.hip): the kernel of steps of
+    single tokens, in either dtype.  max_keys: the most keys any token of the step sees (from the step's longest
+    context and the mask); the other arguments are attention_masked's."""
+    T = q.shape[0]
+    dt = q.dtype
+    if k_pool.dim() != 4 or v_pool.dim() != 4:
+        raise HipLibraryError("k_pool must be [pages, nKV, page, d]")
+    n_pages, nKV, page_size, d = k_pool.shape
+    dv = v_pool.shape[3]
+    _dev(q, "q", None, (T, num_heads * d))
+    _dev(k_pool, "k_pool", dt)
+    _dev(v_pool, "v_pool", dt, tuple(k_pool.shape[:3]) + (dv,))
+    if per_value_head is not None:
+        _dev(per_value_head, "per_value_head", torch.float32, (T, num_heads, nKV, dv))
+        if gate is not None:
+            raise HipLibraryError("per-value-head outputs take no gate: the mix that follows does")
+    else:
+        _dev(out, "out", dt, (T, num_heads * dv))
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        need = num_heads * dv if gate_per_element else num_heads
+        if (not gate.is_cuda or gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != T or gate.shape[1] < need
+                or gate.stride(1) != 1 or gate.stride(0) < need):
+            raise HipLibraryError(f"gate must be [{T}, >= {need}] float32 with unit column stride")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
+    _dev(positions, "positions", torch.int32, (T,))
+    _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
+    _dev(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
+        raise HipLibraryError(f"position {max_position} is beyond the block table {tuple(block_table.shape)}")
+    if bias_slopes is not None:
+        _dev(bias_slopes, "bias_slopes", torch.float32, (num_heads,))
+    if sink is not None:
+        _dev(sink, "sink", torch.float32, (num_heads,))
+    if value_cos is not None:
+        if dv % 2 or value_cos.dim() != 2 or value_cos.shape[1] != dv // 2 or value_sin.shape != value_cos.shape:
+            raise HipLibraryError(f"value tables must be [positions, {dv // 2}]")
+        _dev(value_cos, "value_cos", torch.float32)
+        _dev(value_sin, "value_sin", torch.float32)
+        if max_position >= value_cos.shape[0]:
+            raise HipLibraryError(f"position {max_position} is beyond the rotation tables ({value_cos.shape[0]} positions)")
+    if max_keys < 1 or max_keys > max_position + 1:
+        max_keys = max_position + 1
+    lib = library()
+    runs = lib.alice_attention_split_runs(int(max_keys))
+    work = torch.empty((lib.alice_attention_split_workspace(T, num_heads, nKV, dv, runs, int(per_value_head is not None)),),
+                       dtype=torch.float32, device=q.device)
+    _call("alice_attention_split", q.data_ptr(), dtype_code(dt), k_pool.data_ptr(), v_pool.data_ptr(),
+          None if out is None else out.data_ptr(), None if per_value_head is None else per_value_head.data_ptr(),
+          positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, num_heads, nKV, d, dv,
+          page_size, float(scale), int(window or 0), int(chunk or 0), int(keep_first or 0), int(max_keys),
+          None if bias_slopes is None else bias_slopes.data_ptr(), None if sink is None else sink.data_ptr(),
+          None if value_cos is None else value_cos.data_ptr(), None if value_sin is None else value_sin.data_ptr(),
+          gate_ptr, int(gate_stride), 2 if gate_per_element else 1, float(out_scale), work.data_ptr(), _stream())
 
 
 def mix_heads(a: torch.Tensor, talk: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, *,

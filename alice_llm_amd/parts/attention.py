@@ -243,9 +243,22 @@ class Attention(Part):
         tiled = (not ctx.is_decode and self.softcap is None and not self.precision.full
                  and ops.attention_tiled_supported(act, self.d, self.dv))
 
+        # single tokens: the kernel that splits the keys over blocks, where it takes the head sizes
+        split = (not tiled and ctx.is_decode and self.softcap is None
+                 and ops.attention_split_supported(act, self.nH, self.nKV, self.d, self.dv))
+        if self.chunk is not None:
+            most = min(ctx.max_context, self.chunk)
+        elif self.window is not None:
+            most = min(ctx.max_context, self.window + self.keep_first)
+        else:
+            most = ctx.max_context
+
         def attend(out_, per_, **more):
             if tiled:
                 ops.attention_tiled(q, cache.k, cache.v, out_, ctx, cache.block_table, per_value_head=per_, **common, **more)
+            elif split:
+                ops.attention_split(q, cache.k, cache.v, out_, ctx.positions, ctx.seq_of_token, cache.block_table,
+                                    per_value_head=per_, max_position=ctx.max_position, max_keys=most, **common, **more)
             else:
                 ops.attention_masked(q, cache.k, cache.v, out_, ctx.positions, ctx.seq_of_token, cache.block_table,
                                      per_value_head=per_, softcap=self.softcap, max_position=ctx.max_position,

@@ -150,6 +150,14 @@ def test_window_with_kept_first_positions_sink_and_turned_values(dtype, window, 
                              value_cos=vc, value_sin=vs)
         err = max_err(out.view(n, H, dv), ref[rows])
         assert err < (3e-5 if dtype == "float32" else 8e-2), (rows, err)
+        out2 = torch.empty_like(out)            # the same rows by the kernel that splits the keys over blocks
+        ops.attention_split(q[rows].reshape(n, H * d).contiguous().to(DEV), kp, vp, out2, posd[rows].contiguous(),
+                            seq[rows].contiguous(), bt, num_heads=H, scale=0.5, window=window, keep_first=keep,
+                            max_position=T - 1, max_keys=min(T, window + keep), sink=sink.to(DEV),
+                            gate=gate.to(DEV)[rows][:, :H * dv], gate_per_element=True, out_scale=1.25,
+                            value_cos=vc, value_sin=vs)
+        err = max_err(out2.view(n, H, dv), ref[rows])
+        assert err < (3e-5 if dtype == "float32" else 8e-2), ("split", rows, err)
     if dtype == "bfloat16":                     # the matrix-core kernel of prompts: whole, and in pieces around the edges
         for pieces in _pieces_of(T, [mark + window, keep + window, 64]):
             ctx = _Pieces(pieces, T)
@@ -204,6 +212,13 @@ def test_chunks_distance_term_and_mixed_heads(dtype, chunk, T):
         ops.mix_heads(per, talk.to(DEV), gate.to(DEV)[rows].contiguous(), out, full_precision=dtype == "float32", out_scale=0.75)
         err = max_err(out.view(n, H, dv), ref[rows])
         assert err < (3e-5 if dtype == "float32" else 8e-2), (rows, err)
+        per.fill_(9.0)                          # the same rows by the kernel that splits the keys over blocks
+        ops.attention_split(q[rows].reshape(n, H * d).contiguous().to(DEV), kp, vp, None, posd[rows].contiguous(),
+                            seq[rows].contiguous(), bt, num_heads=H, scale=0.5, chunk=chunk, max_position=T - 1,
+                            max_keys=min(T, chunk), bias_slopes=slopes.float().to(DEV), per_value_head=per)
+        ops.mix_heads(per, talk.to(DEV), gate.to(DEV)[rows].contiguous(), out, full_precision=dtype == "float32", out_scale=0.75)
+        err = max_err(out.view(n, H, dv), ref[rows])
+        assert err < (3e-5 if dtype == "float32" else 8e-2), ("split", rows, err)
     if dtype == "bfloat16":
         for pieces in _pieces_of(T, [last + 1, first, 64]):
             ctx = _Pieces(pieces, T)
