@@ -158,7 +158,7 @@ int alice_qkv_prepare(const void* rows, int rows_dtype, int row_width, const flo
 // x[t, c] += a[t, c] + v[c] (either may be null)
 int alice_add_rows(float* x, const float* a, const float* v, int T, int W, hipStream_t stream);
 // Gated linear attention over a step's tokens, see gla.hip.
-int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, const float* z,
+int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, float* z,
               const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
               int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
               int n_slots, int H, int d, int dv, hipStream_t stream);

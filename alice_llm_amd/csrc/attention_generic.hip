@@ -153,14 +153,13 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
 template <typename T, bool FULL>
 __global__ void mix_heads_kernel(const float* __restrict__ a, const float* __restrict__ talk, const float* __restrict__ gate,
                                  int gate_stride, float out_scale, T* __restrict__ out, int nH, int nKV, int dv) {
-  const int t = blockIdx.x;
-  const int per = nH / nKV;
-  for (int i = threadIdx.x; i < nH * dv; i += blockDim.x) {
-    const int h = i / dv, e = i % dv, c = h / per;
+  const int t = blockIdx.x, h = blockIdx.y;            // a block per (token, head)
+  const int c = h / (nH / nKV);
+  for (int e = threadIdx.x; e < dv; e += blockDim.x) {
     float o = 0.f;
     for (int g = 0; g < nH; ++g) o = fmaf(talk[h * nH + g], a[(((size_t)t * nH + g) * nKV + c) * dv + e], o);
-    if (gate) o *= sigmoid_f(gate[(size_t)t * gate_stride + i], FULL);
-    store_f32(out + (size_t)t * nH * dv, i, o * out_scale);
+    if (gate) o *= sigmoid_f(gate[(size_t)t * gate_stride + h * dv + e], FULL);
+    store_f32(out + ((size_t)t * nH + h) * dv, e, o * out_scale);
   }
 }
 
@@ -227,12 +226,12 @@ extern "C" int alice_attention_masked(const void* q, int dtype, const void* k_po
 extern "C" int alice_mix_heads(const float* a, const float* talk, const float* gate, int gate_stride, float out_scale, void* out,
                                int dtype, int T, int nH, int nKV, int dv, int full_precision, hipStream_t stream) {
   ALICE_CHECK(dtype_ok(dtype), "mix_heads: unknown dtype %d", dtype);
-  ALICE_CHECK(a && talk && out && T >= 0 && nH >= 1 && nKV >= 1 && nH % nKV == 0 && dv >= 1, "mix_heads: bad arguments");
+  ALICE_CHECK(a && talk && out && T >= 0 && nH >= 1 && nH <= 65535 && nKV >= 1 && nH % nKV == 0 && dv >= 1, "mix_heads: bad arguments");
   ALICE_CHECK(gate == nullptr || gate_stride >= nH * dv, "mix_heads: gate rows of %d elements are too short", gate_stride);
   if (T == 0) return 0;
   DISPATCH_DTYPE(dtype, TT, {
-    if (full_precision) mix_heads_kernel<TT, true><<<T, 256, 0, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);
-    else mix_heads_kernel<TT, false><<<T, 256, 0, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);
+    if (full_precision) mix_heads_kernel<TT, true><<<dim3(T, nH), dv > 128 ? 256 : (dv > 64 ? 128 : 64), 0, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);
+    else mix_heads_kernel<TT, false><<<dim3(T, nH), dv > 128 ? 256 : (dv > 64 ? 128 : 64), 0, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);
   });
   ALICE_LAUNCH_CHECK();
   return 0;

@@ -5,8 +5,8 @@
 // and sums.
 //
 // A block of four waves takes 64 consecutive queries of one sequence and one query head, a wave 16 of them.  The
-// keys go through LDS 32 at a time (the next 32 are on their way from memory meanwhile): the key rows as they are,
-// the value rows transposed.  A wave computes the transposed score tile S^T = K Q^T with v_mfma_f32_16x16x32_bf16
+// keys go through LDS 32 at a time, in two buffers (the next 32 are on their way from memory while the waves work
+// on the current ones, and one barrier a step suffices): the key rows as they are, the value rows transposed.  A wave computes the transposed score tile S^T = K Q^T with v_mfma_f32_16x16x32_bf16
 // (keys are the rows, the wave's 16 queries the columns), so that a lane holds eight scores of ONE query: the
 // softmax's maximum and sum are four-lane affairs, and the rounded weights are, as they stand, the second operand
 // of O^T = V^T P^T; the transposed values lie in LDS in the key order in which the score tiles leave the matrix
@@ -55,8 +55,9 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   constexpr int KS = DP / 32, ET = DVP / 16;
   constexpr int KROW = DP + 8;
   constexpr int NKC = DP / 64, NVC = DVP / 64;          // 16-byte pieces of keys / values a thread moves a step
-  __shared__ __align__(16) bf16_t Ks[KT][KROW];
-  __shared__ __align__(16) bf16_t Vt[DVP][VPAD];
+  constexpr int NBUF = (DP + DVP <= 384) ? 2 : 1;        // two buffers where they fit the static LDS limit
+  __shared__ __align__(16) bf16_t Ks[NBUF][KT][KROW];
+  __shared__ __align__(16) bf16_t Vt[NBUF][DVP][VPAD];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
   const int h = blockIdx.y;
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
     }
 #pragma unroll
     for (int n = 0; n < NVC; ++n) {
-      const int id = tid + n * 256, key = id / (DVP / 8), e = (id % (DVP / 8)) * 8, kp = key0 + key;
+      const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8, kp = key0 + key;     // neighbouring lanes: neighbouring keys
       pv[n] = u32x4{0u, 0u, 0u, 0u};
       if (e < DV && kp <= p_last) {
         const int page = bt[kp / a.page_size];
@@ -131,82 +132,89 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   for (int et = 0; et < ET; ++et) oT[et] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
 
-  fetch(0);
-  for (int step = 0; step < n_steps; ++step) {
-    const int key0 = (step < n_first ? step : t_lo + step - n_first) * KT;
-    __syncthreads();                                    // the step before has read its keys and values
+  auto stage = [&](int buf) {                           // what was fetched goes into LDS
 #pragma unroll
     for (int n = 0; n < NKC; ++n) {
       const int id = tid + n * 256, key = id / (DP / 8), dim = (id % (DP / 8)) * 8;
-      *reinterpret_cast<u32x4*>(&Ks[key][dim]) = pk[n];
+      *reinterpret_cast<u32x4*>(&Ks[buf][key][dim]) = pk[n];
     }
 #pragma unroll
     for (int n = 0; n < NVC; ++n) {
-      const int id = tid + n * 256, key = id / (DVP / 8), e = (id % (DVP / 8)) * 8;
+      const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8;
       const int col = ((key & 15) >> 2) * 8 + (key & 3) + 4 * (key >> 4);       // the order of the score tiles' rows
       const uint32_t w[4] = {pv[n][0], pv[n][1], pv[n][2], pv[n][3]};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        Vt[e + 2 * i][col].bits = (uint16_t)(w[i] & 0xffffu);
-        Vt[e + 2 * i + 1][col].bits = (uint16_t)(w[i] >> 16);
+        Vt[buf][e + 2 * i][col].bits = (uint16_t)(w[i] & 0xffffu);
+        Vt[buf][e + 2 * i + 1][col].bits = (uint16_t)(w[i] >> 16);
       }
     }
-    __syncthreads();
-    if (step + 1 < n_steps) fetch(step + 1);
-    if (!wave_on) continue;
+  };
 
-    f32x4 sT[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  for (int step = 0; step < n_steps; ++step) {
+    const int key0 = (step < n_first ? step : t_lo + step - n_first) * KT;
+    const int cur = NBUF == 2 ? (step & 1) : 0;
+    const bool more = step + 1 < n_steps;
+    if (more) fetch(step + 1);
+    if (wave_on) {
+      f32x4 sT[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const u32x4 kf = *reinterpret_cast<const u32x4*>(&Ks[cur][mt * 16 + c][ks * 32 + g * 8]);
+          sT[mt] = mfma32(kf, qf[ks], sT[mt]);
+        }
+      }
+      float sc[8], m_t = -INFINITY;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
-        const u32x4 kf = *reinterpret_cast<const u32x4*>(&Ks[mt * 16 + c][ks * 32 + g * 8]);
-        sT[mt] = mfma32(kf, qf[ks], sT[mt]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kp = key0 + mt * 16 + g * 4 + i;
+          float s = sT[mt][i] * a.scale;
+          if (a.slopes) s = fmaf(slope, (float)(kp - qpos), s);
+          const bool vis = valid && kp <= qpos && (kp >= lo_q || kp < keepf);
+          s = vis ? s : -INFINITY;
+          sc[mt * 4 + i] = s;
+          m_t = fmaxf(m_t, s);
+        }
+      }
+      m_t = fmaxf(m_t, __shfl_xor(m_t, 16, 64));
+      m_t = fmaxf(m_t, __shfl_xor(m_t, 32, 64));
+      if (__ballot(m_t > -INFINITY) != 0ull) {           // else none of the wave's queries sees a key of this block
+        const float m_new = fmaxf(m_run, m_t);
+        float corr = 1.f, sum = 0.f;
+        uint32_t pw[4] = {0u, 0u, 0u, 0u};
+        if (m_new > -INFINITY) {
+          corr = __expf(m_run - m_new);                 // m_run = -inf gives 0
+          float p[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            p[i] = __expf(sc[i] - m_new);
+            sum += p[i];
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pw[i] = pack_bf16x2(p[2 * i], p[2 * i + 1]);
+          m_run = m_new;
+        }
+        l_run = fmaf(l_run, corr, sum);
+        const u32x4 pf = u32x4{pw[0], pw[1], pw[2], pw[3]};
+#pragma unroll
+        for (int et = 0; et < ET; ++et) {
+          const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vt[cur][et * 16 + c][g * 8]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oT[et][i] *= corr;
+          oT[et] = mfma32(vf, pf, oT[et]);
+        }
       }
     }
-    float sc[8], m_t = -INFINITY;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int kp = key0 + mt * 16 + g * 4 + i;
-        float s = sT[mt][i] * a.scale;
-        if (a.slopes) s = fmaf(slope, (float)(kp - qpos), s);
-        const bool vis = valid && kp <= qpos && (kp >= lo_q || kp < keepf);
-        s = vis ? s : -INFINITY;
-        sc[mt * 4 + i] = s;
-        m_t = fmaxf(m_t, s);
-      }
-    }
-    m_t = fmaxf(m_t, __shfl_xor(m_t, 16, 64));
-    m_t = fmaxf(m_t, __shfl_xor(m_t, 32, 64));
-    if (__ballot(m_t > -INFINITY) == 0ull) continue;     // none of the wave's queries sees a key of this block
-    const float m_new = fmaxf(m_run, m_t);
-    float corr = 1.f, sum = 0.f;
-    uint32_t pw[4];
-    if (m_new > -INFINITY) {
-      corr = __expf(m_run - m_new);                     // m_run = -inf gives 0
-      float p[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        p[i] = __expf(sc[i] - m_new);
-        sum += p[i];
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pw[i] = pack_bf16x2(p[2 * i], p[2 * i + 1]);
-      m_run = m_new;
-    } else {
-      pw[0] = pw[1] = pw[2] = pw[3] = 0u;
-    }
-    l_run = fmaf(l_run, corr, sum);
-    const u32x4 pf = u32x4{pw[0], pw[1], pw[2], pw[3]};
-#pragma unroll
-    for (int et = 0; et < ET; ++et) {
-      const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vt[et * 16 + c][g * 8]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) oT[et][i] *= corr;
-      oT[et] = mfma32(vf, pf, oT[et]);
-    }
+    if (NBUF == 1) __syncthreads();                     // one buffer: everybody has read it before it is filled again
+    if (more) stage(NBUF == 2 ? (cur ^ 1) : 0);
+    __syncthreads();
   }
 
   if (!valid) return;

@@ -26,10 +26,17 @@ namespace {
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 __device__ __forceinline__ float silu(float z) { return z / (1.f + expf(-z)); }
 
+// z[t, i] <- sigmoid(z[t, i] + bias[i])^(1 / tau) = exp(logsigmoid(.) / tau), once per key channel for all the blocks
+// that share it, with the full-precision functions on both paths.
+__global__ void gla_decay_kernel(float* __restrict__ z, const float* __restrict__ bias, float inv_tau, long n, int width) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) z[i] = expf(log_sigmoid(z[i] + bias[i % width]) * inv_tau);
+}
+
 template <int CB, int RPT, int TC, typename TW, typename TO>
 __global__ __launch_bounds__(256) void gla_kernel(
     const float* __restrict__ rows, int row_w, int q_col, int k_col, int v_col, int g_col,
-    const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, float q_scale, float out_scale,
+    const float* __restrict__ alpha, float q_scale, float out_scale,
     const TW* __restrict__ norm_w, float eps, TO* __restrict__ out, float* __restrict__ o32,
     const int* __restrict__ cu_seqlens, const int* __restrict__ slots, float* __restrict__ S, int H, int d, int dv) {
   constexpr int RG = 256 / CB;                 // row groups
@@ -55,7 +62,7 @@ __global__ __launch_bounds__(256) void gla_kernel(
     st[i] = (r < d && col_ok) ? Sh[(size_t)r * dv + j] : 0.f;
   }
   const bool finish_here = CB == 64 && gridDim.z == 1;
-  // what this thread fetches for TC tokens: element (t, r) = (idx / DP, idx % DP) of q, k and z; (t, c) of v
+  // what this thread fetches for TC tokens: element (t, r) = (idx / DP, idx % DP) of q, k and the decay; (t, c) of v
   float pq[NL], pk[NL], pz[NL], pv[NV];
   auto fetch = [&](int tc) {
 #pragma unroll
@@ -66,7 +73,7 @@ __global__ __launch_bounds__(256) void gla_kernel(
         const float* row = rows + (size_t)t * row_w;
         pq[n] = row[q_col + h * d + r];
         pk[n] = row[k_col + h * d + r];
-        pz[n] = z[(size_t)t * H * d + h * d + r];
+        pz[n] = alpha[(size_t)t * H * d + h * d + r];
       }
     }
 #pragma unroll
@@ -83,8 +90,7 @@ __global__ __launch_bounds__(256) void gla_kernel(
       const int idx = tid + n * 256, t = idx / DP, r = idx % DP;
       sq[t][r] = pq[n] * q_scale;
       sk[t][r] = pk[n];
-      // rows beyond d hold zeros and stay zero whatever their decay
-      sa[t][r] = r < d ? expf(log_sigmoid(pz[n] + z_bias[h * d + r]) * inv_tau) : 0.f;
+      sa[t][r] = pz[n];                          // (rows beyond d hold zeros and stay zero)
     }
 #pragma unroll
     for (int n = 0; n < NV; ++n) {
@@ -168,10 +174,10 @@ __global__ __launch_bounds__(256) void gla_finish_kernel(const float* __restrict
 
 
 // rows: float32 [T, row_w] with q at q_col (H d), k at k_col (H d), v at v_col (H dv) and the gate at g_col (H dv);
-// z: float32 [T, H d], the decay's pre-activation without its bias z_bias [H d]; S: [n_slots, H, d, dv] float32;
+// z: float32 [T, H d], the decay's pre-activation without its bias z_bias [H d] (overwritten by the decays); S: [n_slots, H, d, dv] float32;
 // out: [T, H dv] in out_dtype, times the constant out_scale; work: float32 [T, H dv] (may be null where (sequences x
 // heads) fill the chip and dv <= 64: then nothing is read from it).
-extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, const float* z,
+extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, float* z,
                          const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
                          int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
                          int n_slots, int H, int d, int dv, hipStream_t stream) {
@@ -188,9 +194,11 @@ extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int
   const bool wide = (long)n_seqs * H * ceil_div(dv, 64) >= 512;
   const bool finish_here = wide && dv <= 64;
   ALICE_CHECK(finish_here || work != nullptr, "gla: this shape needs the workspace");
+  gla_decay_kernel<<<ceil_div((long)T * H * d, 256), 256, 0, stream>>>(z, z_bias, 1.f / tau, (long)T * H * d, H * d);
+  ALICE_LAUNCH_CHECK();
   dim3 grid(n_seqs, H, ceil_div(dv, wide ? 64 : 16));
 #define GO(CB, RPT, TC, TW, TO)                                                                                                  \
-  gla_kernel<CB, RPT, TC, TW, TO><<<grid, 256, 0, stream>>>(rows, row_w, q_col, k_col, v_col, g_col, z, z_bias, 1.f / tau, q_scale, \
+  gla_kernel<CB, RPT, TC, TW, TO><<<grid, 256, 0, stream>>>(rows, row_w, q_col, k_col, v_col, g_col, z, q_scale, \
       out_scale, (const TW*)norm_w, eps, (TO*)out, work, cu_seqlens, slots, S, H, d, dv)
 #define BY_D(TW, TO)                              \
   do {                                            \

@@ -758,7 +758,7 @@ def gla(rows: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, norm_w: torch
         columns, out_scale: float = 1.0) -> None:
     """Gated linear attention over a step (`ctx` gives cu_seqlens, slots, n_seqs): rows float32 [T, width] with q, k,
     v and the gate at `columns` = (q, k, v, g); z float32 [T, heads * d] and z_bias float32 [heads * d]: the decay is
-    sigmoid(z + z_bias)^(1 / tau); S float32 [slots, heads, d, dv]; out [T, heads * dv], times out_scale."""
+    sigmoid(z + z_bias)^(1 / tau), which is left in z; S float32 [slots, heads, d, dv]; out [T, heads * dv], times out_scale."""
     H, d, dv = heads, head_dim, value_head_dim
     T = rows.shape[0]
     _dev(rows, "rows", torch.float32)
