@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const T* __restrict__ q
   constexpr int VEC = 16 / sizeof(T);
   __shared__ __align__(16) float qs[PER][256];
   __shared__ float ps[PER][KEYS];
-  __shared__ int kps[KEYS];
+  __shared__ int rows_of[KEYS];                       // the row of each of the block's keys in kv head 0's part of its page
   __shared__ float wred[4][PER];
   __shared__ __align__(16) float ored[4][256];
 
@@ -72,14 +72,14 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const T* __restrict__ q
   const bool has = tid < nk;
   const int vi = v0 + tid;
   const int kp = has ? (vi < n_first ? vi : start + (vi - n_first)) : 0;
-  kps[tid] = kp;
+  const int row0 = has ? bt[kp / a.page_size] * a.nKV * a.page_size + kp % a.page_size : 0;
+  rows_of[tid] = row0;
   __syncthreads();
   float dot[PER];
 #pragma unroll
   for (int hh = 0; hh < PER; ++hh) dot[hh] = 0.f;
   if (has) {
-    const int page = bt[kp / a.page_size];
-    const T* krow = k_pool + (((size_t)page * a.nKV + kvh) * a.page_size + kp % a.page_size) * d;
+    const T* krow = k_pool + ((size_t)row0 + (size_t)kvh * a.page_size) * d;
     for (int c0 = 0; c0 < d; c0 += 8 * VEC) {           // eight loads on their way at a time
       uint4 w[8];
 #pragma unroll
@@ -150,9 +150,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const T* __restrict__ q
       for (int i = 0; i < VEC; ++i) acc[hh][i] = 0.f;
     if (ec < EC) {
       for (int i = kg; i < nk; i += KG) {
-        const int kpi = kps[i];
-        const int page = bt[kpi / a.page_size];
-        const uint4 w = *reinterpret_cast<const uint4*>(v_pool + (((size_t)page * a.nKV + vh) * a.page_size + kpi % a.page_size) * dv + ec * VEC);
+        const uint4 w = *reinterpret_cast<const uint4*>(v_pool + ((size_t)rows_of[i] + (size_t)vh * a.page_size) * dv + ec * VEC);
         float vf[VEC];
         unpack16<T>(w, vf);
 #pragma unroll

@@ -37,7 +37,7 @@ struct TiledArgs {
   const int* block_table;
   int bt_stride, n_seqs, nH, nKV, d, dv, page_size;
   float scale;
-  int window, chunk, keep_first;
+  int window, chunk, keep_first, page_shift;     // page_shift: log2 of the page size, or -1 where that is no power of two
   const float* slopes;
   const float* sink;
   const float* vcos;
@@ -104,6 +104,12 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
     if (dim < D) qf[ks] = *reinterpret_cast<const u32x4*>(a.q + ((size_t)tq * a.nH + h) * D + dim);
   }
 
+  // the row of position kp in the pools, in rows of one kv head's page (a shift and a mask for the usual page sizes)
+  auto row_of = [&](int kp, int head) -> size_t {
+    const int pi = a.page_shift >= 0 ? kp >> a.page_shift : kp / a.page_size;
+    const int sl = a.page_shift >= 0 ? kp & (a.page_size - 1) : kp % a.page_size;
+    return ((size_t)bt[pi] * a.nKV + head) * a.page_size + sl;
+  };
   u32x4 pk[NKC], pv[NVC];
   auto fetch = [&](int step) {
     const int key0 = (step < n_first ? step : t_lo + step - n_first) * KT;
@@ -111,19 +117,13 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
     for (int n = 0; n < NKC; ++n) {
       const int id = tid + n * 256, key = id / (DP / 8), dim = (id % (DP / 8)) * 8, kp = key0 + key;
       pk[n] = u32x4{0u, 0u, 0u, 0u};
-      if (dim < D && kp <= p_last) {
-        const int page = bt[kp / a.page_size];
-        pk[n] = *reinterpret_cast<const u32x4*>(a.k_pool + (((size_t)page * a.nKV + kvh) * a.page_size + kp % a.page_size) * D + dim);
-      }
+      if (dim < D && kp <= p_last) pk[n] = *reinterpret_cast<const u32x4*>(a.k_pool + row_of(kp, kvh) * D + dim);
     }
 #pragma unroll
     for (int n = 0; n < NVC; ++n) {
       const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8, kp = key0 + key;     // neighbouring lanes: neighbouring keys
       pv[n] = u32x4{0u, 0u, 0u, 0u};
-      if (e < DV && kp <= p_last) {
-        const int page = bt[kp / a.page_size];
-        pv[n] = *reinterpret_cast<const u32x4*>(a.v_pool + (((size_t)page * a.nKV + vh) * a.page_size + kp % a.page_size) * DV + e);
-      }
+      if (e < DV && kp <= p_last) pv[n] = *reinterpret_cast<const u32x4*>(a.v_pool + row_of(kp, vh) * DV + e);
     }
   };
 
@@ -289,8 +289,11 @@ extern "C" int alice_attention_tiled(const void* q, const void* k_pool, const vo
   ALICE_CHECK(((uintptr_t)q & 15) == 0 && ((uintptr_t)k_pool & 15) == 0 && ((uintptr_t)v_pool & 15) == 0 &&
               ((uintptr_t)out & 7) == 0 && ((uintptr_t)out32 & 15) == 0, "attention: operands are not aligned");
   if (T == 0) return 0;
+  int page_shift = -1;
+  for (int b = 0; b < 31; ++b)
+    if (page_size == (1 << b)) page_shift = b;
   TiledArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out, out32, positions, cu_seqlens,
-              block_table, bt_stride, n_seqs, nH, nKV, d, dv, page_size, scale, window, chunk, keep_first, bias_slopes, sink,
+              block_table, bt_stride, n_seqs, nH, nKV, d, dv, page_size, scale, window, chunk, keep_first, page_shift, bias_slopes, sink,
               vrot_cos, vrot_sin, gate, gate_stride, gate_mode, out_scale};
   dim3 grid(ceil_div(T, 64) + n_seqs, nH, out32 ? nKV : 1);
   const int dp = pad_size(d), dvp = pad_size(dv);
