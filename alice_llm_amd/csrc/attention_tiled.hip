@@ -6,7 +6,7 @@
 //
 // A block of four waves takes 64 consecutive queries of one sequence and one query head, a wave 16 of them.  The
 // keys go through LDS 32 at a time, in two buffers (the next 32 are on their way from memory while the waves work
-// on the current ones, and one barrier a step suffices): the key rows as they are, the value rows transposed.  A wave computes the transposed score tile S^T = K Q^T with v_mfma_f32_16x16x32_bf16
+// on the current ones, their page number looked up a step further ahead, and one barrier a step suffices): the key rows as they are, the value rows transposed.  A wave computes the transposed score tile S^T = K Q^T with v_mfma_f32_16x16x32_bf16
 // (keys are the rows, the wave's 16 queries the columns), so that a lane holds eight scores of ONE query: the
 // softmax's maximum and sum are four-lane affairs, and the rounded weights are, as they stand, the second operand
 // of O^T = V^T P^T; the transposed values lie in LDS in the key order in which the score tiles leave the matrix
@@ -65,8 +65,9 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   const int vh = a.out32 ? (int)blockIdx.z : kvh;
   const int D = a.d, DV = a.dv;
 
-  // which 64 queries: the blocks are dealt to the sequences in order, ceil(tokens / 64) each
-  int idx = blockIdx.x, seq = -1, q0 = 0, nq = 0;
+  // which 64 queries: the blocks are dealt to the sequences in order, ceil(tokens / 64) each; the hardware starts
+  // blocks in the order of their index, and the last queries of a sequence have the most keys: they go first
+  int idx = gridDim.x - 1 - blockIdx.x, seq = -1, q0 = 0, nq = 0;
   for (int s = 0; s < a.n_seqs; ++s) {
     const int b = a.cu_seqlens[s], e = a.cu_seqlens[s + 1], nt = (e - b + 63) >> 6;
     if (idx < nt) {
@@ -110,20 +111,33 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
     const int sl = a.page_shift >= 0 ? kp & (a.page_size - 1) : kp % a.page_size;
     return ((size_t)bt[pi] * a.nKV + head) * a.page_size + sl;
   };
+  // With pages of a power of two of at least 32 positions a step's 32 keys lie in one page: its number is looked up
+  // a step ahead of the loads that need it (one dependent load less in a step's way).
+  const bool one_page = a.page_shift >= 5;
+  auto page_of_step = [&](int step) -> int {
+    const int key0 = (step < n_first ? step : t_lo + step - n_first) * KT;
+    return (one_page && step < n_steps) ? bt[key0 >> a.page_shift] : 0;
+  };
   u32x4 pk[NKC], pv[NVC];
-  auto fetch = [&](int step) {
+  auto fetch = [&](int step, int page) {
     const int key0 = (step < n_first ? step : t_lo + step - n_first) * KT;
 #pragma unroll
     for (int n = 0; n < NKC; ++n) {
       const int id = tid + n * 256, key = id / (DP / 8), dim = (id % (DP / 8)) * 8, kp = key0 + key;
       pk[n] = u32x4{0u, 0u, 0u, 0u};
-      if (dim < D && kp <= p_last) pk[n] = *reinterpret_cast<const u32x4*>(a.k_pool + row_of(kp, kvh) * D + dim);
+      if (dim < D && kp <= p_last) {
+        const size_t row = one_page ? ((size_t)page * a.nKV + kvh) * a.page_size + (kp & (a.page_size - 1)) : row_of(kp, kvh);
+        pk[n] = *reinterpret_cast<const u32x4*>(a.k_pool + row * D + dim);
+      }
     }
 #pragma unroll
     for (int n = 0; n < NVC; ++n) {
       const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8, kp = key0 + key;     // neighbouring lanes: neighbouring keys
       pv[n] = u32x4{0u, 0u, 0u, 0u};
-      if (e < DV && kp <= p_last) pv[n] = *reinterpret_cast<const u32x4*>(a.v_pool + row_of(kp, vh) * DV + e);
+      if (e < DV && kp <= p_last) {
+        const size_t row = one_page ? ((size_t)page * a.nKV + vh) * a.page_size + (kp & (a.page_size - 1)) : row_of(kp, vh);
+        pv[n] = *reinterpret_cast<const u32x4*>(a.v_pool + row * DV + e);
+      }
     }
   };
 
@@ -151,14 +165,16 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
     }
   };
 
-  fetch(0);
+  fetch(0, page_of_step(0));
+  int page_next = page_of_step(1);
   stage(0);
   __syncthreads();
   for (int step = 0; step < n_steps; ++step) {
     const int key0 = (step < n_first ? step : t_lo + step - n_first) * KT;
     const int cur = NBUF == 2 ? (step & 1) : 0;
     const bool more = step + 1 < n_steps;
-    if (more) fetch(step + 1);
+    if (more) fetch(step + 1, page_next);
+    page_next = page_of_step(step + 2);
     if (wave_on) {
       f32x4 sT[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
