@@ -133,7 +133,7 @@ int alice_attention_tiled(const void* q, const void* k_pool, const void* v_pool,
                           int T, int n_seqs, int nH, int nKV, int d, int dv, int page_size, float scale, int window,
                           int chunk, int keep_first, const float* bias_slopes, const float* sink,
                           const float* vrot_cos, const float* vrot_sin, const float* gate, int gate_stride,
-                          int gate_mode, float out_scale, hipStream_t stream);
+                          int gate_mode, float out_scale, int heads_per_wave, hipStream_t stream);
 // alice_attention_masked's result for single tokens with the keys split over blocks (attention_split.hip), either
 // dtype, 32-bit arithmetic; max_keys: the most keys any token of the step sees; work: alice_attention_split_workspace
 // floats (runs = alice_attention_split_runs(max_keys)).

@@ -4,7 +4,9 @@
 // and the per-value-head outputs that a mix of the heads' weights needs.  bfloat16 operands, 32-bit scores, softmax
 // and sums.
 //
-// A block of four waves takes 64 consecutive queries of one sequence and one query head, a wave 16 of them.  The
+// A block of four waves takes 64 consecutive queries of one sequence and HPW query heads of one kv head's group
+// (1; 2 or 4 at the caller's wish), a wave 16 of the queries for all of those heads: a staged block of keys and
+// values, and every fragment a wave reads of it, serves all of them.  The
 // keys go through LDS 32 at a time, in two buffers (the next 32 are on their way from memory while the waves work
 // on the current ones, their page number looked up a step further ahead, and one barrier a step suffices): the key rows as they are, the value rows transposed.  A wave computes the transposed score tile S^T = K Q^T with v_mfma_f32_16x16x32_bf16
 // (keys are the rows, the wave's 16 queries the columns), so that a lane holds eight scores of ONE query: the
@@ -50,7 +52,7 @@ struct TiledArgs {
 constexpr int KT = 32;        // keys a step
 constexpr int VPAD = 40;      // row length of the transposed values in LDS (32 keys and a pad against bank conflicts)
 
-template <int DP, int DVP>
+template <int DP, int DVP, int HPW>
 __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   constexpr int KS = DP / 32, ET = DVP / 16;
   constexpr int KROW = DP + 8;
@@ -60,8 +62,8 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   __shared__ __align__(16) bf16_t Vt[NBUF][DVP][VPAD];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
-  const int h = blockIdx.y;
-  const int per = a.nH / a.nKV, kvh = h / per;
+  const int h0 = blockIdx.y * HPW;                      // the wave's heads: h0 .. h0 + HPW - 1, of one kv head
+  const int per = a.nH / a.nKV, kvh = h0 / per;
   const int vh = a.out32 ? (int)blockIdx.z : kvh;
   const int D = a.d, DV = a.dv;
 
@@ -87,7 +89,9 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   const int qpos = a.positions[tq];
   const int keepf = (a.window > 0 && a.chunk == 0) ? a.keep_first : 0;
   const int lo_q = a.chunk > 0 ? (qpos / a.chunk) * a.chunk : (a.window > 0 ? qpos + 1 - a.window : 0);
-  const float slope = a.slopes ? a.slopes[h] : 0.f;
+  float slope[HPW];
+#pragma unroll
+  for (int hh = 0; hh < HPW; ++hh) slope[hh] = a.slopes ? a.slopes[h0 + hh] : 0.f;
 
   // the key blocks: the first n_first of the kept positions, then t_lo .. t_hi
   const int lo = a.chunk > 0 ? (p_first / a.chunk) * a.chunk : (a.window > 0 ? max(0, p_first + 1 - a.window) : 0);
@@ -97,12 +101,15 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   const int n_steps = n_first + t_hi - t_lo + 1;
 
   // the wave's queries as the second operand of S^T = K Q^T: column c, dimensions ks*32 + g*8 .. +7
-  u32x4 qf[KS];
+  u32x4 qf[HPW][KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int dim = ks * 32 + g * 8;
-    qf[ks] = u32x4{0u, 0u, 0u, 0u};
-    if (dim < D) qf[ks] = *reinterpret_cast<const u32x4*>(a.q + ((size_t)tq * a.nH + h) * D + dim);
+  for (int hh = 0; hh < HPW; ++hh) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int dim = ks * 32 + g * 8;
+      qf[hh][ks] = u32x4{0u, 0u, 0u, 0u};
+      if (dim < D) qf[hh][ks] = *reinterpret_cast<const u32x4*>(a.q + ((size_t)tq * a.nH + h0 + hh) * D + dim);
+    }
   }
 
   // the row of position kp in the pools, in rows of one kv head's page (a shift and a mask for the usual page sizes)
@@ -141,10 +148,15 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
     }
   };
 
-  f32x4 oT[ET];
+  f32x4 oT[HPW][ET];
+  float m_run[HPW], l_run[HPW];
 #pragma unroll
-  for (int et = 0; et < ET; ++et) oT[et] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
+  for (int hh = 0; hh < HPW; ++hh) {
+    m_run[hh] = -INFINITY;
+    l_run[hh] = 0.f;
+#pragma unroll
+    for (int et = 0; et < ET; ++et) oT[hh][et] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   auto stage = [&](int buf) {                           // what was fetched goes into LDS
 #pragma unroll
@@ -176,55 +188,70 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
     if (more) fetch(step + 1, page_next);
     page_next = page_of_step(step + 2);
     if (wave_on) {
-      f32x4 sT[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+      f32x4 sT[HPW][2];
+#pragma unroll
+      for (int hh = 0; hh < HPW; ++hh) sT[hh][0] = sT[hh][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
           const u32x4 kf = *reinterpret_cast<const u32x4*>(&Ks[cur][mt * 16 + c][ks * 32 + g * 8]);
-          sT[mt] = mfma32(kf, qf[ks], sT[mt]);
+#pragma unroll
+          for (int hh = 0; hh < HPW; ++hh) sT[hh][mt] = mfma32(kf, qf[hh][ks], sT[hh][mt]);
         }
       }
-      float sc[8], m_t = -INFINITY;
+      // which of the lane's eight keys its query sees (the same for every head)
+      bool vis[8];
+      bool any = false;
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kp = key0 + mt * 16 + g * 4 + i;
-          float s = sT[mt][i] * a.scale;
-          if (a.slopes) s = fmaf(slope, (float)(kp - qpos), s);
-          const bool vis = valid && kp <= qpos && (kp >= lo_q || kp < keepf);
-          s = vis ? s : -INFINITY;
-          sc[mt * 4 + i] = s;
-          m_t = fmaxf(m_t, s);
-        }
+      for (int j = 0; j < 8; ++j) {
+        const int kp = key0 + (j >> 2) * 16 + g * 4 + (j & 3);
+        vis[j] = valid && kp <= qpos && (kp >= lo_q || kp < keepf);
+        any = any || vis[j];
       }
-      m_t = fmaxf(m_t, __shfl_xor(m_t, 16, 64));
-      m_t = fmaxf(m_t, __shfl_xor(m_t, 32, 64));
-      if (__ballot(m_t > -INFINITY) != 0ull) {           // else none of the wave's queries sees a key of this block
-        const float m_new = fmaxf(m_run, m_t);
-        float corr = 1.f, sum = 0.f;
-        uint32_t pw[4] = {0u, 0u, 0u, 0u};
-        if (m_new > -INFINITY) {
-          corr = __expf(m_run - m_new);                 // m_run = -inf gives 0
-          float p[8];
+      if (__ballot(any) != 0ull) {                       // else none of the wave's queries sees a key of this block
+        u32x4 pf[HPW];
+        float corr[HPW];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            p[i] = __expf(sc[i] - m_new);
-            sum += p[i];
+        for (int hh = 0; hh < HPW; ++hh) {
+          float sc[8], m_t = -INFINITY;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            float sv = sT[hh][j >> 2][j & 3] * a.scale;
+            if (a.slopes) sv = fmaf(slope[hh], (float)(key0 + (j >> 2) * 16 + g * 4 + (j & 3) - qpos), sv);
+            sc[j] = vis[j] ? sv : -INFINITY;
+            m_t = fmaxf(m_t, sc[j]);
           }
+          m_t = fmaxf(m_t, __shfl_xor(m_t, 16, 64));
+          m_t = fmaxf(m_t, __shfl_xor(m_t, 32, 64));
+          const float m_new = fmaxf(m_run[hh], m_t);
+          float sum = 0.f;
+          uint32_t pw[4] = {0u, 0u, 0u, 0u};
+          corr[hh] = 1.f;
+          if (m_new > -INFINITY) {
+            corr[hh] = __expf(m_run[hh] - m_new);       // m_run = -inf gives 0
+            float p[8];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) pw[i] = pack_bf16x2(p[2 * i], p[2 * i + 1]);
-          m_run = m_new;
+            for (int j = 0; j < 8; ++j) {
+              p[j] = __expf(sc[j] - m_new);
+              sum += p[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) pw[j] = pack_bf16x2(p[2 * j], p[2 * j + 1]);
+            m_run[hh] = m_new;
+          }
+          l_run[hh] = fmaf(l_run[hh], corr[hh], sum);
+          pf[hh] = u32x4{pw[0], pw[1], pw[2], pw[3]};
         }
-        l_run = fmaf(l_run, corr, sum);
-        const u32x4 pf = u32x4{pw[0], pw[1], pw[2], pw[3]};
 #pragma unroll
         for (int et = 0; et < ET; ++et) {
           const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vt[cur][et * 16 + c][g * 8]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) oT[et][i] *= corr;
-          oT[et] = mfma32(vf, pf, oT[et]);
+          for (int hh = 0; hh < HPW; ++hh) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oT[hh][et][i] *= corr[hh];
+            oT[hh][et] = mfma32(vf, pf[hh], oT[hh][et]);
+          }
         }
       }
     }
@@ -234,45 +261,49 @@ __global__ __launch_bounds__(256) void attn_tiled_kernel(TiledArgs a) {
   }
 
   if (!valid) return;
-  float l_tot = l_run;
-  l_tot += __shfl_xor(l_tot, 16, 64);
-  l_tot += __shfl_xor(l_tot, 32, 64);
-  float factor = 1.f;
-  if (a.sink) {                                         // one more term of the denominator, without a value
-    const float sk = a.sink[h];
-    const float m_fin = fmaxf(m_run, sk);
-    factor = __expf(m_run - m_fin);
-    l_tot = fmaf(l_tot, factor, __expf(sk - m_fin));
-  }
-  const float inv = l_tot > 0.f ? factor / l_tot : 0.f;
   const size_t t = (size_t)tq;
 #pragma unroll
-  for (int et = 0; et < ET; ++et) {
-    const int e = et * 16 + g * 4;
-    if (e >= DV) continue;
-    float o[4];
+  for (int hh = 0; hh < HPW; ++hh) {
+    const int h = h0 + hh;
+    float l_tot = l_run[hh];
+    l_tot += __shfl_xor(l_tot, 16, 64);
+    l_tot += __shfl_xor(l_tot, 32, 64);
+    float factor = 1.f;
+    if (a.sink) {                                       // one more term of the denominator, without a value
+      const float sk = a.sink[h];
+      const float m_fin = fmaxf(m_run[hh], sk);
+      factor = __expf(m_run[hh] - m_fin);
+      l_tot = fmaf(l_tot, factor, __expf(sk - m_fin));
+    }
+    const float inv = l_tot > 0.f ? factor / l_tot : 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = oT[et][i] * inv;
-    if (a.vcos) {                                       // the pairs (e, e + 1) turned back by the query's position
+    for (int et = 0; et < ET; ++et) {
+      const int e = et * 16 + g * 4;
+      if (e >= DV) continue;
+      float o[4];
 #pragma unroll
-      for (int i = 0; i < 4; i += 2) {
-        const float cs = a.vcos[(size_t)qpos * (DV >> 1) + ((e + i) >> 1)], sn = a.vsin[(size_t)qpos * (DV >> 1) + ((e + i) >> 1)];
-        const float u = o[i], v = o[i + 1];
-        o[i] = fmaf(u, cs, __fmul_rn(v, sn));
-        o[i + 1] = fmaf(v, cs, -__fmul_rn(u, sn));
+      for (int i = 0; i < 4; ++i) o[i] = oT[hh][et][i] * inv;
+      if (a.vcos) {                                     // the pairs (e, e + 1) turned back by the query's position
+#pragma unroll
+        for (int i = 0; i < 4; i += 2) {
+          const float cs = a.vcos[(size_t)qpos * (DV >> 1) + ((e + i) >> 1)], sn = a.vsin[(size_t)qpos * (DV >> 1) + ((e + i) >> 1)];
+          const float u = o[i], v = o[i + 1];
+          o[i] = fmaf(u, cs, __fmul_rn(v, sn));
+          o[i + 1] = fmaf(v, cs, -__fmul_rn(u, sn));
+        }
       }
-    }
-    if (a.out32) {
-      *reinterpret_cast<f32x4*>(a.out32 + ((t * a.nH + h) * a.nKV + vh) * DV + e) = f32x4{o[0], o[1], o[2], o[3]};
-      continue;
-    }
+      if (a.out32) {
+        *reinterpret_cast<f32x4*>(a.out32 + ((t * a.nH + h) * a.nKV + vh) * DV + e) = f32x4{o[0], o[1], o[2], o[3]};
+        continue;
+      }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (a.gate) o[i] *= sigmoid_f(a.gate[t * a.gate_stride + (a.gate_mode == 2 ? h * DV + e + i : h)], false);
-      o[i] *= a.out_scale;
+      for (int i = 0; i < 4; ++i) {
+        if (a.gate) o[i] *= sigmoid_f(a.gate[t * a.gate_stride + (a.gate_mode == 2 ? h * DV + e + i : h)], false);
+        o[i] *= a.out_scale;
+      }
+      uint2 pkd = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+      *reinterpret_cast<uint2*>(a.out + (t * a.nH + h) * DV + e) = pkd;
     }
-    uint2 pkd = {pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
-    *reinterpret_cast<uint2*>(a.out + (t * a.nH + h) * DV + e) = pkd;
   }
 }
 
@@ -286,13 +317,14 @@ extern "C" int alice_attention_tiled_supported(int d, int dv) {
 
 // q: bfloat16 [T, nH d]; pools: bfloat16 [pages, nKV, page, d / dv] row-major; out: bfloat16 [T, nH dv], or out32:
 // float32 [T, nH, nKV, dv] (then nothing goes to out and no gate is applied); gate: float32 rows.  The step's tokens
-// are those of n_seqs sequences in order (cu_seqlens), each at consecutive positions.
+// are those of n_seqs sequences in order (cu_seqlens), each at consecutive positions.  heads_per_wave: 0 is the
+// launcher's choice (1); 2 or 4 ask for that many heads of a group a wave.
 extern "C" int alice_attention_tiled(const void* q, const void* k_pool, const void* v_pool, void* out, float* out32,
                                      const int* positions, const int* cu_seqlens, const int* block_table, int bt_stride,
                                      int T, int n_seqs, int nH, int nKV, int d, int dv, int page_size, float scale, int window,
                                      int chunk, int keep_first, const float* bias_slopes, const float* sink,
                                      const float* vrot_cos, const float* vrot_sin, const float* gate, int gate_stride,
-                                     int gate_mode, float out_scale, hipStream_t stream) {
+                                     int gate_mode, float out_scale, int heads_per_wave, hipStream_t stream) {
   ALICE_CHECK(alice_attention_tiled_supported(d, dv), "attention: head sizes %d and %d are outside this kernel's range (multiples of 8 up to 256)", d, dv);
   ALICE_CHECK(q && k_pool && v_pool && (out || out32) && positions && cu_seqlens && block_table, "attention: a pointer is missing");
   ALICE_CHECK(T >= 0 && n_seqs >= 1 && nH >= 1 && nKV >= 1 && nH % nKV == 0, "attention: bad head counts nH=%d nKV=%d", nH, nKV);
@@ -311,9 +343,29 @@ extern "C" int alice_attention_tiled(const void* q, const void* k_pool, const vo
   TiledArgs a{(const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, (bf16_t*)out, out32, positions, cu_seqlens,
               block_table, bt_stride, n_seqs, nH, nKV, d, dv, page_size, scale, window, chunk, keep_first, page_shift, bias_slopes, sink,
               vrot_cos, vrot_sin, gate, gate_stride, gate_mode, out_scale};
-  dim3 grid(ceil_div(T, 64) + n_seqs, nH, out32 ? nKV : 1);
   const int dp = pad_size(d), dvp = pad_size(dv);
-#define GO(DP, DVP) attn_tiled_kernel<DP, DVP><<<grid, 256, 0, stream>>>(a)
+  // Heads of a kv head's group a wave: one.  Two or four (each staged key block and every fragment read of it then
+  // serves them all) measured slower at head sizes of 128, for want of registers (one wave a SIMD instead of three):
+  // one prompt of 2,048 tokens 86 us with one head a wave, 108 with two; eight prompts 552 against 744 with four.
+  const int per = nH / nKV;
+  int hpw = 1;
+  if (heads_per_wave > 0) {                             // the caller's choice (tests)
+    ALICE_CHECK((heads_per_wave == 1 || heads_per_wave == 2 || heads_per_wave == 4) && per % heads_per_wave == 0 &&
+                (heads_per_wave == 1 || (dp <= 128 && dvp <= 128)),
+                "attention: %d heads a wave do not divide the group of %d, or the head sizes are beyond 128", heads_per_wave, per);
+    hpw = heads_per_wave;
+  }
+  dim3 grid(ceil_div(T, 64) + n_seqs, nH / hpw, out32 ? nKV : 1);
+#define GO(DP, DVP)                                                         \
+  do {                                                                      \
+    if constexpr (DP <= 128 && DVP <= 128) {                                \
+      if (hpw == 4) attn_tiled_kernel<DP, DVP, 4><<<grid, 256, 0, stream>>>(a);      \
+      else if (hpw == 2) attn_tiled_kernel<DP, DVP, 2><<<grid, 256, 0, stream>>>(a); \
+      else attn_tiled_kernel<DP, DVP, 1><<<grid, 256, 0, stream>>>(a);               \
+    } else {                                                                \
+      attn_tiled_kernel<DP, DVP, 1><<<grid, 256, 0, stream>>>(a);           \
+    }                                                                       \
+  } while (0)
 #define BY_DV(DP)                     \
   do {                                \
     if (dvp == 64) GO(DP, 64);        \

@@ -58,7 +58,7 @@ def _declare(lib) -> None:
         "alice_attention_generic": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, P],
         "alice_head_gate": [P, I, P, I, I, I, I, P],
         "alice_attention_masked": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, F, I, P, I, I, P, I, I, F, I, I, P, P, P, P, P],
-        "alice_attention_tiled": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, I, P, P, P, P, P, I, I, F, P],
+        "alice_attention_tiled": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, I, P, P, P, P, P, I, I, F, I, P],
         "alice_attention_tiled_supported": [I, I],
         "alice_attention_split": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, I, P, P, P, P, P, I, I, F, P, P],
         "alice_attention_split_supported": [I, I, I, I, I],
@@ -548,10 +548,11 @@ def attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                     chunk: Optional[int] = None, keep_first: int = 0, bias_slopes: Optional[torch.Tensor] = None,
                     sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, gate_per_element: bool = False,
                     out_scale: float = 1.0, value_cos: Optional[torch.Tensor] = None, value_sin: Optional[torch.Tensor] = None,
-                    per_value_head: Optional[torch.Tensor] = None) -> None:
+                    per_value_head: Optional[torch.Tensor] = None, heads_per_wave: int = 0) -> None:
     """attention_masked's result for bfloat16 prompts by the matrix-core kernel over the row-major cache (see
     attention_tiled.hip): `ctx` gives positions, cu_seqlens and the step's sizes; every sequence's tokens stand at
-    consecutive positions.  The other arguments are attention_masked's."""
+    consecutive positions.  heads_per_wave: how many heads of a kv head's group a wave takes (0: the launcher's
+    choice by the step's size; 1, 2 or 4).  The other arguments are attention_masked's."""
     T = q.shape[0]
     if k_pool.dim() != 4 or v_pool.dim() != 4:
         raise HipLibraryError("k_pool must be [pages, nKV, page, d]")
@@ -597,7 +598,7 @@ def attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
           int(window or 0), int(chunk or 0), int(keep_first or 0), None if bias_slopes is None else bias_slopes.data_ptr(),
           None if sink is None else sink.data_ptr(), None if value_cos is None else value_cos.data_ptr(),
           None if value_sin is None else value_sin.data_ptr(), gate_ptr, int(gate_stride), 2 if gate_per_element else 1,
-          float(out_scale), _stream())
+          float(out_scale), int(heads_per_wave), _stream())
 
 
 def attention_split_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int, value_head_dim: int) -> bool:

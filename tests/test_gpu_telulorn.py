@@ -159,16 +159,16 @@ def test_window_with_kept_first_positions_sink_and_turned_values(dtype, window, 
         err = max_err(out2.view(n, H, dv), ref[rows])
         assert err < (3e-5 if dtype == "float32" else 8e-2), ("split", rows, err)
     if dtype == "bfloat16":                     # the matrix-core kernel of prompts: whole, and in pieces around the edges
-        for pieces in _pieces_of(T, [mark + window, keep + window, 64]):
+        for hpw, pieces in [(w, p) for w in (1, 2) for p in _pieces_of(T, [mark + window, keep + window, 64])]:
             ctx = _Pieces(pieces, T)
             n = ctx.rows.numel()
             out = torch.empty(n, H * dv, dtype=dt, device=DEV)
             ops.attention_tiled(q[ctx.rows].reshape(n, H * d).contiguous().to(DEV), kp, vp, out, ctx, bt.expand(ctx.n_seqs, -1).contiguous(),
                                 num_heads=H, scale=0.5, window=window, keep_first=keep, sink=sink.to(DEV),
                                 gate=gate.to(DEV)[ctx.rows][:, :H * dv], gate_per_element=True, out_scale=1.25,
-                                value_cos=vc, value_sin=vs)
+                                value_cos=vc, value_sin=vs, heads_per_wave=hpw)
             err = max_err(out.view(n, H, dv), ref[ctx.rows])
-            assert err < 8e-2, (len(pieces), err)
+            assert err < 8e-2, (hpw, len(pieces), err)
     if mark + window < T:
         assert (ref[mark + window - 1] - ref[mark + window]).abs().max() > 0.3          # the markers do show
     if keep and keep + window < T:
@@ -180,8 +180,9 @@ def test_window_with_kept_first_positions_sink_and_turned_values(dtype, window, 
 def test_chunks_distance_term_and_mixed_heads(dtype, chunk, T):
     """A marker key at the last position of a chunk: seen by that position alone, not by the first query of the next
     chunk; another at a chunk's first position, seen to the chunk's end.  The distance term is taken off the scores,
-    the heads' weights are mixed by a matrix far from the identity, and every head keeps its own kv head's values."""
-    H, G, d, dv, page = 6, 3, 16, 24, 64
+    the heads' weights are mixed by a matrix far from the identity, and every head keeps its own kv head's values.  The
+    prompt kernel is run with one, two and four heads of a group a wave."""
+    H, G, d, dv, page = 8, 2, 16, 24, 64
     dt = torch.float32 if dtype == "float32" else torch.bfloat16
     q, k, v = rnd(T, H, d, seed=1), rnd(T, G, d, seed=2), rnd(T, G, dv, seed=3)
     gate = rnd(T, H * dv, seed=4, scale=2.0)
@@ -220,16 +221,17 @@ def test_chunks_distance_term_and_mixed_heads(dtype, chunk, T):
         err = max_err(out.view(n, H, dv), ref[rows])
         assert err < (3e-5 if dtype == "float32" else 8e-2), ("split", rows, err)
     if dtype == "bfloat16":
-        for pieces in _pieces_of(T, [last + 1, first, 64]):
+        for hpw, pieces in [(w, p) for w in (1, 2, 4) for p in _pieces_of(T, [last + 1, first, 64])]:
             ctx = _Pieces(pieces, T)
             n = ctx.rows.numel()
             per = torch.empty(n, H, G, dv, dtype=torch.float32, device=DEV)
             out = torch.empty(n, H * dv, dtype=dt, device=DEV)
             ops.attention_tiled(q[ctx.rows].reshape(n, H * d).contiguous().to(DEV), kp, vp, None, ctx, bt.expand(ctx.n_seqs, -1).contiguous(),
-                                num_heads=H, scale=0.5, chunk=chunk, bias_slopes=slopes.float().to(DEV), per_value_head=per)
+                                num_heads=H, scale=0.5, chunk=chunk, bias_slopes=slopes.float().to(DEV), per_value_head=per,
+                                heads_per_wave=hpw)
             ops.mix_heads(per, talk.to(DEV), gate.to(DEV)[ctx.rows].contiguous(), out, full_precision=False, out_scale=0.75)
             err = max_err(out.view(n, H, dv), ref[ctx.rows])
-            assert err < 8e-2, (len(pieces), err)
+            assert err < 8e-2, (hpw, len(pieces), err)
     if last + 1 < T:
         assert (ref[last] - ref[last + 1]).abs().max() > 0.3
 
