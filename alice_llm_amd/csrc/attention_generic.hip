@@ -163,6 +163,25 @@ __global__ void mix_heads_kernel(const float* __restrict__ a, const float* __res
   }
 }
 
+// The same with a block per (token, kv head): the kv head's column of all heads' outputs goes through LDS once and
+// serves the group's heads (dynamic LDS of nH * dv floats).
+template <typename T, bool FULL>
+__global__ void mix_heads_group_kernel(const float* __restrict__ a, const float* __restrict__ talk, const float* __restrict__ gate,
+                                       int gate_stride, float out_scale, T* __restrict__ out, int nH, int nKV, int dv) {
+  extern __shared__ float col[];                       // [nH][dv]
+  const int t = blockIdx.x, c = blockIdx.y, per = nH / nKV;
+  for (int i = threadIdx.x; i < nH * dv; i += blockDim.x)
+    col[i] = a[(((size_t)t * nH + i / dv) * nKV + c) * dv + i % dv];
+  __syncthreads();
+  for (int i = threadIdx.x; i < per * dv; i += blockDim.x) {
+    const int h = c * per + i / dv, e = i % dv;
+    float o = 0.f;
+    for (int g = 0; g < nH; ++g) o = fmaf(talk[h * nH + g], col[g * dv + e], o);
+    if (gate) o *= sigmoid_f(gate[(size_t)t * gate_stride + h * dv + e], FULL);
+    store_f32(out + ((size_t)t * nH + h) * dv, e, o * out_scale);
+  }
+}
+
 }  // namespace
 
 static int attention_generic_launch(const void* q, int dtype, const void* k_pool, const void* v_pool, void* out,
@@ -229,6 +248,15 @@ extern "C" int alice_mix_heads(const float* a, const float* talk, const float* g
   ALICE_CHECK(a && talk && out && T >= 0 && nH >= 1 && nH <= 65535 && nKV >= 1 && nH % nKV == 0 && dv >= 1, "mix_heads: bad arguments");
   ALICE_CHECK(gate == nullptr || gate_stride >= nH * dv, "mix_heads: gate rows of %d elements are too short", gate_stride);
   if (T == 0) return 0;
+  if ((size_t)nH * dv * sizeof(float) <= 48 * 1024 && nKV <= 65535) {      // the column fits LDS: a block per (token, kv head)
+    const size_t lds = (size_t)nH * dv * sizeof(float);
+    DISPATCH_DTYPE(dtype, TT, {
+      if (full_precision) mix_heads_group_kernel<TT, true><<<dim3(T, nKV), 256, lds, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);
+      else mix_heads_group_kernel<TT, false><<<dim3(T, nKV), 256, lds, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);
+    });
+    ALICE_LAUNCH_CHECK();
+    return 0;
+  }
   DISPATCH_DTYPE(dtype, TT, {
     if (full_precision) mix_heads_kernel<TT, true><<<dim3(T, nH), dv > 128 ? 256 : (dv > 64 ? 128 : 64), 0, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);
     else mix_heads_kernel<TT, false><<<dim3(T, nH), dv > 128 ? 256 : (dv > 64 ? 128 : 64), 0, stream>>>(a, talk, gate, gate_stride, out_scale, (TT*)out, nH, nKV, dv);

@@ -321,8 +321,8 @@ def telulorn_configs(size, vocab=32768, window=1024):
     heads = {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5}
     mlp = {"kind": "dense", "ff": z["ff"]}
     par = {"type": "parallel", "mlp": mlp,
-           "mixer": {"left": dict(heads, mask={"size": window}), "left_scale": 1.2, "right_scale": 1.1,
-                     "right": {"heads": z["mheads"], "dim": z["mdim"], "vdim": z["mvdim"], "tau": 16.0, "rank": 64}}}
+           "mixer": {"left": dict(heads, mask={"size": window}), "left_scale": 1.0, "right_scale": 0.9,
+                     "right": {"heads": z["mheads"], "dim": z["mdim"], "vdim": z["mvdim"], "tau": 8.0, "rank": 64}}}
     att = {"type": "attention", "mlp": mlp,
            "mixer": dict(heads, mask={"size": window, "keep_first": 64}, rot={"base": 10000.0, "dims": z["dim"] // 2})}
     return {"architecture": "Telulorn", "vocab": vocab, "width": z["width"], "norm": {"eps": 1e-6},

@@ -244,8 +244,8 @@ def novotar_pair(name: str, dtype: str, seed: int = 0, device="cuda"):
 #    window and a chunk longer than a page; tau 1; both side factors 1.
 # C: sizes that suit the matrix cores; a loop over every layer run three times; one kv head; a chunk of exactly a
 #    page; kept first positions that reach into the second page; value heads of the recurrence wider than 64.
-# D: an attention layer first; a loop over the first layer alone; a layer without any mask and one whose window
-#    keeps no first positions; keys of the recurrence wider than 128; three query heads a kv head.
+# D: an attention layer first; a loop over the first layer alone; a layer without any mask or rotation and one whose
+#    window keeps no first positions; keys of the recurrence wider than 128; three query heads a kv head.
 def _tl_par(left, right, mlp, ls=1.0, rs=1.0):
     return {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": ls, "right_scale": rs}, "mlp": mlp}
 
@@ -286,7 +286,7 @@ def _tl_d():
     le = {"heads": 3, "kv_heads": 1, "dim": 24, "vdim": 24, "scale": 0.2}
     ri = {"heads": 1, "dim": 136, "vdim": 24, "tau": 8.0, "rank": 3}
     at = {"heads": 6, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.25, "mask": {"size": 33}, "rot": {"base": 50.0, "dims": 8}}
-    free = {k: v for k, v in at.items() if k != "mask"}
+    free = {k: v for k, v in at.items() if k not in ("mask", "rot")}      # no mask and no rotation at all
     mlp = {"kind": "dense", "ff": 80}
     return {"architecture": "Telulorn", "vocab": 61, "width": 48, "norm": {"eps": 1e-6},
             "layers": [{"type": "attention", "mixer": at, "mlp": mlp}, _tl_par(le, ri, mlp, 1.2, 1.0),

@@ -44,6 +44,7 @@ def test_defaults_and_absent_keys():
     raw = TELULORN["tl-d"]()
     plan = alice.config_from_dict(raw).plan()
     assert plan.layers[2].mixer.args["window"] is None and plan.layers[2].mixer.args["keep_first"] == 0
+    assert plan.layers[2].mixer.args["position"] is None and len(plan.positions) == 1
     assert plan.layers[0].mixer.args["keep_first"] == 0 and plan.layers[0].mixer.args["window"] == 33
     assert plan.layers[1].mixer.args["sides"][0].args["chunk"] is None
     no_loop = alice.config_from_dict(TELULORN["tl-b"]()).plan()
