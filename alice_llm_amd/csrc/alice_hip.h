@@ -161,7 +161,7 @@ int alice_add_rows(float* x, const float* a, const float* v, int T, int W, hipSt
 int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, float* z,
               const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
               int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
-              int n_slots, int H, int d, int dv, hipStream_t stream);
+              int n_slots, int H, int d, int dv, int columns, hipStream_t stream);
 int alice_head_gate(void* out, int out_layout, const void* gate, int gate_stride, int T, int nH, int d, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 // out may be absent when splits > 1: the splits are then left in `parts`, [B][nH][splits][ALICE_ATTN_PARTS_HEAD + d]

@@ -13,8 +13,8 @@
 // TC at a time: q, k and the decays of TC tokens are put there by all threads (the next TC tokens' operands are
 // already on their way from memory), every thread then updates its rows token by token, with no barrier between
 // the tokens, and keeps its TC partial read-outs, which meet in LDS once per TC tokens and are added up in the
-// order of the row groups.  CB is 64 where (sequences x heads) fill the chip, 16 otherwise (more blocks, fewer rows
-// a thread).  Which rows belong to the sequence and which state row is its own are read on the device
+// order of the row groups.  CB is 64 where (sequences x heads) fill the chip, else 16, or 8 where even that leaves CUs
+// without a block (more blocks, fewer rows a thread).  Which rows belong to the sequence and which state row is its own are read on the device
 // (cu_seqlens, slots), so a launch depends on sizes only.  With CB = 64 and dv <= 64 the head's norm and gate are
 // finished by the block itself; otherwise o is left in a float32 workspace for gla_finish_kernel (the norm needs
 // every column of a head).
@@ -176,12 +176,13 @@ __global__ __launch_bounds__(256) void gla_finish_kernel(const float* __restrict
 // rows: float32 [T, row_w] with q at q_col (H d), k at k_col (H d), v at v_col (H dv) and the gate at g_col (H dv);
 // z: float32 [T, H d], the decay's pre-activation without its bias z_bias [H d] (overwritten by the decays); S: [n_slots, H, d, dv] float32;
 // out: [T, H dv] in out_dtype, times the constant out_scale; work: float32 [T, H dv] (may be null where (sequences x
-// heads) fill the chip and dv <= 64: then nothing is read from it).
+// heads) fill the chip and dv <= 64: then nothing is read from it).  columns: value columns a block (0: by the step's size).
 extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int g_col, float* z,
                          const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
                          int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
-                         int n_slots, int H, int d, int dv, hipStream_t stream) {
+                         int n_slots, int H, int d, int dv, int columns, hipStream_t stream) {
   ALICE_CHECK(dtype_ok(w_dtype) && dtype_ok(out_dtype), "gla: unknown dtype");
+  ALICE_CHECK(columns == 0 || columns == 8 || columns == 16 || columns == 64, "gla: %d value columns a block are not built (8, 16, 64; 0: by the step's size)", columns);
   ALICE_CHECK(rows && z && z_bias && norm_w && out && cu_seqlens && slots && S, "gla: a pointer is missing");
   ALICE_CHECK(T >= 0 && n_seqs >= 0 && n_slots >= 1 && H >= 1 && d >= 1 && dv >= 1, "gla: bad sizes");
   ALICE_CHECK(d <= 256, "gla: key size %d is beyond 256, the range of this kernel", d);
@@ -191,12 +192,15 @@ extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int
   ALICE_CHECK(H <= 65535 && dv <= 65535 * 16, "gla: too many heads for one launch");
   if (T == 0 || n_seqs == 0) return 0;
   // 64 columns a block where that fills the chip, else 16 (four times the blocks)
-  const bool wide = (long)n_seqs * H * ceil_div(dv, 64) >= 512;
+  // value columns a block: 64 where that fills the chip twice, else 16, else 8 where 16 leave CUs without a block
+  int cb = columns;
+  if (cb == 0) cb = (long)n_seqs * H * ceil_div(dv, 64) >= 512 ? 64 : ((long)n_seqs * H * ceil_div(dv, 16) >= 256 ? 16 : 8);
+  const bool wide = cb == 64;
   const bool finish_here = wide && dv <= 64;
   ALICE_CHECK(finish_here || work != nullptr, "gla: this shape needs the workspace");
   gla_decay_kernel<<<ceil_div((long)T * H * d, 256), 256, 0, stream>>>(z, z_bias, 1.f / tau, (long)T * H * d, H * d);
   ALICE_LAUNCH_CHECK();
-  dim3 grid(n_seqs, H, ceil_div(dv, wide ? 64 : 16));
+  dim3 grid(n_seqs, H, ceil_div(dv, cb));
 #define GO(CB, RPT, TC, TW, TO)                                                                                                  \
   gla_kernel<CB, RPT, TC, TW, TO><<<grid, 256, 0, stream>>>(rows, row_w, q_col, k_col, v_col, g_col, z, q_scale, \
       out_scale, (const TW*)norm_w, eps, (TO*)out, work, cu_seqlens, slots, S, H, d, dv)
@@ -206,10 +210,13 @@ extern "C" int alice_gla(const float* rows, int row_w, int q_col, int k_col, int
       if (d <= 64) GO(64, 16, 8, TW, TO);         \
       else if (d <= 128) GO(64, 32, 4, TW, TO);   \
       else GO(64, 64, 4, TW, TO);                 \
-    } else {                                      \
+    } else if (cb == 16) {                        \
       if (d <= 64) GO(16, 4, 16, TW, TO);         \
       else if (d <= 128) GO(16, 8, 16, TW, TO);   \
       else GO(16, 16, 8, TW, TO);                 \
+    } else {                                      \
+      if (d <= 128) GO(8, 4, 16, TW, TO);         \
+      else GO(8, 8, 8, TW, TO);                   \
     }                                             \
   } while (0)
   if (w_dtype == DT_F32 && out_dtype == DT_F32) BY_D(float, float);

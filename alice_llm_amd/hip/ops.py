@@ -66,7 +66,7 @@ def _declare(lib) -> None:
         "alice_mix_heads": [P, P, P, I, F, P, I, I, I, I, I, I, P],
         "alice_qkv_prepare": [P, I, I, P, P, P, P, I, P, P, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "alice_add_rows": [P, P, P, I, I, P],
-        "alice_gla": [P, I, I, I, I, I, P, P, F, F, F, P, I, F, P, I, P, P, P, P, I, I, I, I, I, I, P],
+        "alice_gla": [P, I, I, I, I, I, P, P, F, F, F, P, I, F, P, I, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
         "alice_argmax": [P, P, P, P, I, I, P],
@@ -756,10 +756,11 @@ GLA_MAX_KEY_DIM = 256       # the largest key size the gated linear attention ke
 
 def gla(rows: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, norm_w: torch.Tensor, out: torch.Tensor, ctx,
         S: torch.Tensor, *, heads: int, head_dim: int, value_head_dim: int, tau: float, q_scale: float, eps: float,
-        columns, out_scale: float = 1.0) -> None:
+        columns, out_scale: float = 1.0, columns_per_block: int = 0) -> None:
     """Gated linear attention over a step (`ctx` gives cu_seqlens, slots, n_seqs): rows float32 [T, width] with q, k,
     v and the gate at `columns` = (q, k, v, g); z float32 [T, heads * d] and z_bias float32 [heads * d]: the decay is
-    sigmoid(z + z_bias)^(1 / tau), which is left in z; S float32 [slots, heads, d, dv]; out [T, heads * dv], times out_scale."""
+    sigmoid(z + z_bias)^(1 / tau), which is left in z; S float32 [slots, heads, d, dv]; out [T, heads * dv], times out_scale.  columns_per_block: 0 lets the launcher
+    choose by the step's size; 8, 16 or 64 fix the value columns a block."""
     H, d, dv = heads, head_dim, value_head_dim
     T = rows.shape[0]
     _dev(rows, "rows", torch.float32)
@@ -778,7 +779,7 @@ def gla(rows: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, norm_w: torch
     _call("alice_gla", rows.data_ptr(), rows.shape[1], q_col, k_col, v_col, g_col, z.data_ptr(), z_bias.data_ptr(), float(tau),
           float(q_scale), float(out_scale), norm_w.data_ptr(), dtype_code(norm_w.dtype), float(eps), out.data_ptr(), dtype_code(out.dtype),
           _opt(work, "work"), ctx.cu_seqlens.data_ptr(), ctx.slots.data_ptr(), S.data_ptr(), T, int(ctx.n_seqs), int(n_slots),
-          H, d, dv, _stream())
+          H, d, dv, int(columns_per_block), _stream())
 
 
 def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:

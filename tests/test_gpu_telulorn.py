@@ -305,11 +305,12 @@ class _Ctx:
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cb", [0, 8, 16, 64])
 @pytest.mark.parametrize("H,d,dv", [(2, 16, 32), (3, 12, 20), (1, 136, 24), (2, 64, 128), (1, 256, 70)])
-def test_gated_linear_attention_over_two_steps_on_shuffled_state_rows(dtype, H, d, dv):
+def test_gated_linear_attention_over_two_steps_on_shuffled_state_rows(dtype, H, d, dv, cb):
     """Three unequal sequences (one of a single token) on state rows in another order, then a second step of single
     tokens and a piece from the state the first step left; decays from fast to none; the state rows of other
-    slots untouched."""
+    slots untouched.  With every number of value columns a block that is built, and the launcher's own choice."""
     dt = torch.float32 if dtype == "float32" else torch.bfloat16
     tau, eps = 4.0, 1e-5
     cols = (3, 3 + H * d, 5 + 2 * H * d, 5 + 2 * H * d + H * dv)          # a layout with gaps
@@ -325,7 +326,7 @@ def test_gated_linear_attention_over_two_steps_on_shuffled_state_rows(dtype, H, 
         rows, z = rnd(T, width, seed=10 + step), rnd(T, H * d, seed=20 + step, scale=2.0)
         out = torch.empty(T, H * dv, dtype=dt, device=DEV)
         ops.gla(rows.to(DEV), z.to(DEV), bias.to(DEV), w.to(DEV), out, _Ctx(lens, slots), S, heads=H, head_dim=d,
-                value_head_dim=dv, tau=tau, q_scale=d ** -0.5, eps=eps, columns=cols, out_scale=1.5)
+                value_head_dim=dv, tau=tau, q_scale=d ** -0.5, eps=eps, columns=cols, out_scale=1.5, columns_per_block=cb)
         at = 0
         for i, n in enumerate(lens):
             ref, states[i] = _gla_plain(rows[at:at + n], z[at:at + n], bias, w, H, d, dv, tau, eps, cols, states[i])
